@@ -28,6 +28,7 @@ class CacheGroup:
     layers: tuple[int, ...]
     pages: tuple = ()
     window: int | None = None
+    keep_first: int = 0     # with a window: positions at a sequence's start that are kept too
 
 
 @dataclass(frozen=True)
@@ -214,7 +215,8 @@ class CacheManager:
             if table is None:
                 continue
             upto = min(self._first_live_block(g, num_computed), len(table))
-            for i in range(self._released[g][request_id], upto):
+            kept = self.blocks_needed(self.groups[g].keep_first)   # pages of the kept first positions
+            for i in range(max(self._released[g][request_id], kept), upto):
                 if table[i] != RELEASED:
                     p.release(table[i])
                     table[i] = RELEASED

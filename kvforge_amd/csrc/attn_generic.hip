@@ -11,7 +11,9 @@
 // so that a lane ends up with four neighbouring keys of one query row: the running maximum and
 // sum of a row are a lane's own, the probabilities stay in registers and are the right-hand
 // operand of O^T += V^T P as they are.  Key j is visible to the query at position p iff j <= p,
-// j < context length and, with a window w > 0, j > p - w.  Scores are scaled after the dot
+// j < context length and, with a window w > 0, j > p - w or j < keep (the first `keep` keys of a
+// sequence stay visible behind the window; the walk over the key tiles then has two pieces, the
+// tiles of the kept keys and the tiles from the window's first key on).  Scores are scaled after the dot
 // product; with `slopes` (one number per q head) slopes[h] * (j - p) is added to them, a bias by
 // distance.  The order of every sum is fixed by the positions alone.
 //
@@ -24,6 +26,7 @@ constexpr int ITEM_ROWS = 64;   // rows per work item: four waves of 16
 
 struct AttnArgs {
   int H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs;
+  int keep;  // with a window: the first `keep` keys of a sequence stay visible
   float scale;
   const float* slopes;  // null, or one number per q head: slopes[h] * (key - query position) is added to a score
 };
@@ -121,14 +124,27 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
 
   const bool quads = a.block_size % 4 == 0;
   const int chunks = D / 8;
-  for (int t0 = (lo / BK) * BK; t0 <= hi; t0 += BK) {
+  // tiles counted in one unbroken range: those of the kept keys, then those from `lo` on
+  const int keep = a.window > 0 ? a.keep : 0;
+  int tc_first = (lo / BK) * BK, tc_last = hi, kept_end = 0, gap = 0;
+  if (keep > 0) {
+    const int ke = ((keep + BK - 1) / BK) * BK;
+    if (tc_first > ke) {
+      kept_end = ke;
+      gap = tc_first - ke;
+      tc_last = hi - gap;
+    }
+    tc_first = 0;
+  }
+  for (int tc = tc_first; tc <= tc_last; tc += BK) {
+    const int t0 = tc >= kept_end ? tc + gap : tc;
     // ---- keys of the tile
     __syncthreads();   // the values of the tile before have been used
     for (int ch = tid; ch < BK * chunks; ch += 256) {
       const int c = ch / chunks, k8 = (ch - c * chunks) * 8;
       const int j = t0 + c;
       float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      if (j >= lo && j <= hi) {
+      if ((j >= lo || j < keep) && j <= hi) {
         const int blk = j / a.block_size;
         const int page = blk < a.table_stride ? table[blk] : -1;
         if (page >= 0 && page < a.num_blocks)
@@ -139,7 +155,7 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
       *reinterpret_cast<float4*>(&KVs[c * KLD + k8 + 4]) = make_float4(v[4], v[5], v[6], v[7]);
     }
     __syncthreads();
-    const bool mine = t0 <= hi_w && t0 + BK > lo_w;   // the same in all lanes of the wave
+    const bool mine = t0 <= hi_w && (t0 + BK > lo_w || t0 < keep);   // the same in all lanes of the wave
     f32x4 p[ST];
     float corr = 1.f;
     if (mine) {
@@ -159,7 +175,7 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
         for (int v = 0; v < 4; ++v) {
           const int j = t0 + 16 * st + 4 * g4 + v;
           bool vis = row_ok && j <= pos && j < ctx;
-          if (a.window > 0) vis = vis && (j > pos - a.window);
+          if (a.window > 0) vis = vis && (j > pos - a.window || j < keep);
           sc[v] = vis ? fmaf(slope, static_cast<float>(j - pos), sc[v] * a.scale) : -INFINITY;
           tmax = fmaxf(tmax, sc[v]);
         }
@@ -196,7 +212,7 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
         const int e = idx / (BK / 4), c = (idx - e * (BK / 4)) * 4;
         const int j = t0 + c;
         f32x4 v = f32x4{0.f, 0.f, 0.f, 0.f};
-        if (j + 3 >= lo && j <= hi) {
+        if ((j + 3 >= lo || j < keep) && j <= hi) {
           const int blk = j / a.block_size;
           const int page = blk < a.table_stride ? table[blk] : -1;
           if (page >= 0 && page < a.num_blocks) {
@@ -204,7 +220,7 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
                       (j - blk * a.block_size));
 #pragma unroll
             for (int x = 0; x < 4; ++x)
-              if (j + x < lo || j + x > hi) v[x] = 0.f;
+              if ((j + x < lo && j + x >= keep) || j + x > hi) v[x] = 0.f;
           }
         }
         *reinterpret_cast<f32x4*>(&KVs[e * VLD + c]) = v;
@@ -214,7 +230,7 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
         const int e = idx / BK, c = idx - e * BK;
         const int j = t0 + c;
         float v = 0.f;
-        if (j >= lo && j <= hi) {
+        if ((j >= lo || j < keep) && j <= hi) {
           const int blk = j / a.block_size;
           const int page = blk < a.table_stride ? table[blk] : -1;
           if (page >= 0 && page < a.num_blocks)
@@ -280,6 +296,7 @@ constexpr int DEC_WAVES = 4, DEC_KEYS = 64;
 
 struct DecodeArgs {
   int H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs, splits;
+  int keep;  // as in AttnArgs
   float scale;
   const float* slopes;  // as in AttnArgs
 };
@@ -310,8 +327,21 @@ __global__ __launch_bounds__(DEC_WAVES * KVF_WAVE) void attn_decode_kernel(
   int lo = 0;
   if (a.window > 0 && pos - a.window + 1 > 0) lo = pos - a.window + 1;
   // blocks of 64 keys from the block that holds `lo`; this cut takes blocks [b_lo, b_hi)
-  const int first = lo / DEC_KEYS;
-  const int n_blocks = ctx > 0 ? pos / DEC_KEYS - first + 1 : 0;
+  // (counted in one unbroken range: the blocks of the kept keys, then those from `lo` on)
+  const int keep = a.window > 0 ? a.keep : 0;
+  int first = lo / DEC_KEYS, kept_blocks = 0, gap = 0;
+  int n_blocks = ctx > 0 ? pos / DEC_KEYS - first + 1 : 0;
+  if (keep > 0 && ctx > 0) {
+    const int kb = (keep + DEC_KEYS - 1) / DEC_KEYS;
+    if (first > kb) {
+      kept_blocks = kb;
+      gap = first - kb;
+      n_blocks += kb;
+    } else {
+      n_blocks += first;
+    }
+    first = 0;
+  }
   const int per_cut = (n_blocks + a.splits - 1) / a.splits;
   const int b_lo = first + cut * per_cut, b_hi = min(first + n_blocks, b_lo + per_cut);
   const int* table = block_table + static_cast<size_t>(seq_ok ? seq : 0) * a.table_stride;
@@ -334,9 +364,10 @@ __global__ __launch_bounds__(DEC_WAVES * KVF_WAVE) void attn_decode_kernel(
     for (int i = 0; i < DQ; ++i) acc[g][i] = 0.f;
   }
   const bool quads = a.block_size % 4 == 0;
-  for (int b = b_lo + wave; b < b_hi; b += DEC_WAVES) {
+  for (int bc = b_lo + wave; bc < b_hi; bc += DEC_WAVES) {
+    const int b = bc >= kept_blocks && keep > 0 ? bc + gap : bc;
     const int j = b * DEC_KEYS + lane;  // this lane's key
-    const bool vis = j >= lo && j <= pos;
+    const bool vis = (j >= lo || j < keep) && j <= pos;
     // the page of every key of the context, visible or not: the values of four neighbouring keys
     // are read together further down, and a hidden one among them only has probability zero
     int page = -1;
@@ -545,14 +576,14 @@ KVF_EXPORT int kvf_attn_generic_decode(int dtype, const void* q, const void* k_p
                                        void* out, float* part_acc, float* part_ml, int num_seqs,
                                        int H, int KV, int d, int block_size, int num_blocks,
                                        int table_stride, int q_stride, int o_stride, int window,
-                                       int n_seqs, int splits, float scale, const float* slopes,
-                                       hipStream_t s) {
+                                       int keep, int n_seqs, int splits, float scale,
+                                       const float* slopes, hipStream_t s) {
   if (num_seqs <= 0) return 0;
-  if (d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || splits < 1 ||
+  if (keep < 0 || d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || splits < 1 ||
       (splits > 1 && (!part_acc || !part_ml)) || block_size <= 0)
     return static_cast<int>(hipErrorInvalidValue);
   DecodeArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
-               splits, scale, slopes};
+               splits, keep, scale, slopes};
   if (dtype == 0)
     return launch_decode<float>(q, k_pages, v_pages, block_table, seq_ids, cu_q, ctx_lens, out,
                                 part_acc, part_ml, num_seqs, a, s);
@@ -569,13 +600,13 @@ KVF_EXPORT int kvf_attn_generic(int dtype, const void* q, const void* k_pages, c
                                 const int* block_table, const int* cu_q, const int* ctx_lens,
                                 const int* work, int num_work, void* out, int H, int KV, int d,
                                 int block_size, int num_blocks, int table_stride, int q_stride,
-                                int o_stride, int window, int n_seqs, float scale,
+                                int o_stride, int window, int keep, int n_seqs, float scale,
                                 const float* slopes, hipStream_t s) {
-  if (d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || !work || block_size <= 0 ||
+  if (keep < 0 || d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || !work || block_size <= 0 ||
       q_stride % 4 != 0 || o_stride % 4 != 0)
     return static_cast<int>(hipErrorInvalidValue);
   AttnArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
-             scale, slopes};
+             keep, scale, slopes};
   if (dtype == 0)
     return launch<float>(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, out, a, s);
   if (dtype == 1)

@@ -18,7 +18,13 @@
 //   bytes.  Probabilities go from the first product's accumulators to the second product's
 //   operand by a rounding to bf16 alone; softmax itself is fp32.
 // Key j is visible to a query at position p iff j <= p, j < context length and, with a window
-// w > 0, j > p - w.  Scores are scaled after the dot product.
+// w > 0, j > p - w or j < keep (the first `keep` keys of a sequence stay visible behind the
+// window).  Scores are scaled after the dot product.
+// A windowed walk with kept keys has two pieces, the blocks that hold keys 0 .. keep - 1 and the
+// blocks from the window's first key on.  The loops below count blocks in one unbroken range
+// (`Walk`: the kept blocks first, the window's blocks right behind them) and turn a count into
+// a key where they look up pages, load fragments or mask, so their pipelines do not know of
+// the gap.
 // With `slopes` (one number per q head) a score also gets slopes[h] * (j - p), a bias by distance;
 // the kernels are instantiated with and without it, so that attention without it pays nothing.
 // The softmax reference of a row (what is subtracted before exp) is raised only when some score
@@ -63,11 +69,33 @@ constexpr float LOG2E = 1.4426950408889634f;
 
 struct MArgs {
   int H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits;
+  int keep;        // with a window: the first `keep` keys of a sequence stay visible
   int kv_fastest;  // query runs: the kv head is the grid's fastest index (see kvf_attn_mfma_prefill)
   float scale;
   unsigned bs_magic;  // floor(2^32 / bs) + 1: key / bs == mulhi(key, bs_magic) while key * bs < 2^32
   const float* slopes;  // null, or one number per q head: slopes[h] * (key - query position) is added to a score
 };
+
+// A walk over the blocks of 32 keys that a range of rows sees: blocks counted from `first` up to
+// `last` (in keys, multiples of 32; none if last < first) stand for the keys `at(count)`.
+struct Walk {
+  int kept_end, gap, first, last;
+  __device__ __forceinline__ int at(int kb) const { return kb >= kept_end ? kb + gap : kb; }
+};
+// lo, hi: first and last key the rows see through the window (hi < 0: none)
+__device__ __forceinline__ Walk walk_of(const MArgs& a, int lo, int hi) {
+  Walk w{0, 0, (lo / 32) * 32, hi};
+  if (a.window > 0 && a.keep > 0 && hi >= 0) {
+    const int kept_end = ((a.keep + 31) / 32) * 32;
+    if (w.first > kept_end) {
+      w.kept_end = kept_end;
+      w.gap = w.first - kept_end;
+      w.last = hi - w.gap;
+    }
+    w.first = 0;
+  }
+  return w;
+}
 
 // Position of a key in its page table: (page table entry, slot in the page)
 __device__ __forceinline__ int block_of(const MArgs& a, int key) {
@@ -163,6 +191,7 @@ template <int RT> struct Rows {
   int tok[RT], head[RT];
   int first[RT];       // first visible key of the row
   unsigned span[RT];   // visible keys are first .. first + span; a row that is none has first < 0
+  int keep[RT];        // and the keys below this (kept behind a window; 0 for a row that is none)
   int pos[RT];         // the row's own position; with slope2, only for kernels with BIAS
   float slope2[RT];    // the head's slope in log2 units
 };
@@ -197,7 +226,7 @@ __device__ __forceinline__ void block_update(const bf16x8 (&kf)[2][(DT + 1) / 2]
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key = kb + 8 * kg + 4 * t + r;
-          const bool vis = static_cast<unsigned>(key - rows.first[rt]) <= rows.span[rt];
+          const bool vis = static_cast<unsigned>(key - rows.first[rt]) <= rows.span[rt] || key < rows.keep[rt];
           s[rt][t][r] = vis ? s[rt][t][r] : -INFINITY;
         }
   }
@@ -275,6 +304,7 @@ __device__ __forceinline__ void setup_rows(const bf16_t* q, const MArgs& a, int 
       const int first = a.window > 0 && pos - a.window + 1 > 0 ? pos - a.window + 1 : 0;
       rows.first[rt] = rows.ok[rt] ? first : -1;
       rows.span[rt] = rows.ok[rt] ? static_cast<unsigned>(pos - first) : 0u;
+      rows.keep[rt] = rows.ok[rt] && a.window > 0 ? min(a.keep, pos + 1) : 0;
       rows.pos[rt] = pos;
       rows.slope2[rt] = a.slopes && rows.ok[rt] ? a.slopes[rows.head[rt]] * LOG2E : 0.f;
     }
@@ -350,6 +380,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
     if (a.window > 0 && p_lo - a.window + 1 > 0) lo_g = p_lo - a.window + 1;
   }
   const float scale2 = a.scale * LOG2E;
+  const int keep_w = a.window > 0 ? a.keep : 0;
 
   float m_ref[RT], l_run[RT];
   f32x4 acc[RT][DT];
@@ -403,11 +434,14 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
     // Every load below reads a valid address whatever the block (a key past the context reads
     // the table's last entry and page 0, and counts for nothing), so none of them sits in a
     // branch and the compiler can count them.
+    const Walk wk = walk_of(a, lo_g, hi_g);
     auto locate = [&](int kb, Lookup& l) {
+      kb = wk.at(kb);
 #pragma unroll
       for (int i = 0; i < FPW; ++i) l.page[i] = page_of_key(pg, a, kb + key_off[i]);
     };
     auto fetch = [&](int kb, const Lookup& l, Stage& st) {
+      kb = wk.at(kb);
 #pragma unroll
       for (int i = 0; i < FPW; ++i) {
         const int key = kb + key_off[i];
@@ -427,7 +461,8 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
       }
     };
     auto work_on = [&](int kb, int buf) {
-      if (kb <= hi_w && kb + 31 >= lo_w) {
+      kb = wk.at(kb);
+      if (kb <= hi_w && (kb + 31 >= lo_w || kb < keep_w)) {
         bf16x8 kf[2][DC], vf[DT];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -440,7 +475,8 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
         block_update<DT, RT, BIAS>(kf, vf, qf, rows, kb, kg, edge, scale2, m_ref, l_run, acc);
       }
     };
-    const int kb_first = (lo_g / 32) * 32;
+    const int kb_first = wk.first;
+    hi_g = wk.last;
     Stage sa;
     Lookup la;
     if constexpr (DEEP) {
@@ -496,9 +532,11 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
       }
     }
   } else {
-    PageRef pk[2] = {k_page(pg, a, (lo_w / 32) * 32, 0), k_page(pg, a, (lo_w / 32) * 32, 1)};
-    PageRef pv = v_page(pg, a, (lo_w / 32) * 32);
-    for (int kb = (lo_w / 32) * 32; kb <= hi_w; kb += 32) {
+    const Walk wk = walk_of(a, lo_w, hi_w);
+    PageRef pk[2] = {k_page(pg, a, wk.at(wk.first), 0), k_page(pg, a, wk.at(wk.first), 1)};
+    PageRef pv = v_page(pg, a, wk.at(wk.first));
+    for (int kc = wk.first; kc <= wk.last; kc += 32) {
+      const int kb = wk.at(kc);
       uint4 kr[2][DC], vr[DT];
       int kl[2][DC], vl;
 #pragma unroll
@@ -507,9 +545,9 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
         for (int c = 0; c < DC; ++c) kr[t][c] = k_fragment<DT>(pg, a, kb, t, c, pk[t], kl[t][c]);
 #pragma unroll
       for (int t = 0; t < DT; ++t) vr[t] = v_fragment(pg, a, kb, t, pv, vl);
-      pk[0] = k_page(pg, a, kb + 32, 0);
-      pk[1] = k_page(pg, a, kb + 32, 1);
-      pv = v_page(pg, a, kb + 32);
+      pk[0] = k_page(pg, a, wk.at(kc + 32), 0);
+      pk[1] = k_page(pg, a, wk.at(kc + 32), 1);
+      pv = v_page(pg, a, wk.at(kc + 32));
       bf16x8 kf[2][DC], vf[DT];
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -580,8 +618,9 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
   // Blocks of 32 keys go round the waves of all cuts in turn: cut z, wave w take blocks
   // z * NW + w, then every (NW * splits)-th.  Without a window the first block is known before
   // the context length has arrived.
-  const int kb0 = (lo / 32) * 32;
-  const int kb_end = hi + 1;
+  const Walk wk = walk_of(a, lo, hi);
+  const int kb0 = wk.first;
+  const int kb_end = wk.last + 1;
   const int turn = (static_cast<int>(blockIdx.z) * NW + wave) * 32;
   const int kb_begin = kb0 + turn;
   const int STEP = 32 * NW * a.splits;
@@ -601,11 +640,13 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
   Raw A, B;
   PageRef pA[3], pB[3];
   auto locate = [&](int kb, PageRef (&p)[3]) {
+    kb = wk.at(kb);
     p[0] = k_page(pg, a, kb, 0);
     p[1] = k_page(pg, a, kb, 1);
     p[2] = v_page(pg, a, kb);
   };
   auto fetch = [&](int kb, const PageRef (&p)[3], Raw& r) {
+    kb = wk.at(kb);
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -614,6 +655,7 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
     for (int t = 0; t < DT; ++t) r.v[t] = v_fragment(pg, a, kb, t, p[2], r.vl);
   };
   auto consume = [&](int kb, const Raw& r) {
+    kb = wk.at(kb);
     bf16x8 kf[2][DC], vf[DT];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -893,9 +935,10 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
                                      const int* block_table, const int* cu_q, const int* ctx_lens,
                                      const int* work, int num_work, int rows_per_item, void* out, int H, int KV, int d,
                                      int bs, int nb, int table_stride, int q_stride, int o_stride,
-                                     int window, int n_seqs, float scale, const float* slopes,
+                                     int window, int keep, int n_seqs, float scale, const float* slopes,
                                      hipStream_t s) {
   if (num_work <= 0) return 0;
+  if (keep < 0) return static_cast<int>(hipErrorInvalidValue);
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0)
     return static_cast<int>(hipErrorInvalidValue);
   const int row_tiles = rows_per_item / (WAVES * 16);
@@ -904,7 +947,7 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
   // workgroups go to consecutive XCDs, so with eight kv heads every XCD walks the keys and values
   // of one head and finds them in its own L2 after the first workgroup has brought them in.
   const int kv_fastest = num_work <= 65535 ? 1 : 0;
-  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, kv_fastest, scale, magic_of(bs), slopes};
+  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, keep, kv_fastest, scale, magic_of(bs), slopes};
   const dim3 grid = kv_fastest ? dim3(KV, num_work) : dim3(num_work, KV);
   switch (d / 16) {
 #define GO(DT) \
@@ -923,13 +966,14 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
                                     const int* ctx_lens, void* out, float* part_acc, float* part_ml,
                                     int num_seqs, int H, int KV, int d, int bs, int nb,
                                     int table_stride, int q_stride, int o_stride, int window,
-                                    int n_seqs, int splits, float scale, const float* slopes,
+                                    int keep, int n_seqs, int splits, float scale, const float* slopes,
                                     hipStream_t s) {
   if (num_seqs <= 0) return 0;
+  if (keep < 0) return static_cast<int>(hipErrorInvalidValue);
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0 || splits < 1 ||
       splits > KVF_WAVE || (splits > 1 && (!part_acc || !part_ml)))
     return static_cast<int>(hipErrorInvalidValue);
-  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, 0, scale, magic_of(bs), slopes};
+  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, keep, 0, scale, magic_of(bs), slopes};
   const int G = H / KV, chunks = (G + 15) / 16;
   if (num_seqs > 65535) return static_cast<int>(hipErrorInvalidValue);
   const dim3 grid(KV * chunks, num_seqs, splits);

@@ -246,6 +246,8 @@ KVF_EXPORT int kvf_silu_mul_bf16(const void* gu, void* out, int m, int inter, in
 // matrix cores contracts over).  With write_kv == 0 only q is rotated.
 struct RopeArgs {
   int H, KV, d, rot, table_len, block_size, table_stride, num_blocks, write_kv, n_seqs;
+  int row_len;  // elements from one token's row to the next: (H + 2 KV) d, or more when the
+                // product that made the rows has further columns behind q, k and v
 };
 
 template <typename T>
@@ -257,7 +259,7 @@ __global__ void rope_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__
   const int n = blockIdx.x;
   const int p = positions[n];
   const int half = a.rot / 2;
-  T* row = qkv + static_cast<size_t>(n) * (a.H + 2 * a.KV) * a.d;
+  T* row = qkv + static_cast<size_t>(n) * a.row_len;
   const bool pos_ok = p >= 0 && p < a.table_len;
   const float* cs = cos_t + static_cast<size_t>(pos_ok ? p : 0) * half;
   const float* sn = sin_t + static_cast<size_t>(pos_ok ? p : 0) * half;
@@ -365,7 +367,7 @@ __global__ __launch_bounds__(256) void rope_kvwrite_tile_kernel(
   }
   __syncthreads();
   // blockIdx.y names a share of the row: of its q and k vectors, and of its V columns
-  const int row_len = (a.H + 2 * a.KV) * a.d;
+  const int row_len = a.row_len;
   const int qk_vecs = (a.H + a.KV) * a.d / 8;
   const int qk_share = (qk_vecs + gridDim.y - 1) / gridDim.y;
   const int qk_begin = blockIdx.y * qk_share;
@@ -438,7 +440,7 @@ static int rope_launch(void* qkv, const int* positions, const int* seq_of_token,
                        const float* sin_t, const int* block_table, void* k_pages, void* v_pages,
                        int n, RopeArgs a, hipStream_t s) {
   if (n <= 0) return 0;
-  if (a.d % 8 == 0 && a.rot % 8 == 0) {
+  if (a.d % 8 == 0 && a.rot % 8 == 0 && a.row_len % 8 == 0) {
     // few tiles: several workgroups share a tile's row, so that the chip has work
     const int tiles = (n + ROPE_TILE - 1) / ROPE_TILE;
     int shares = tiles >= 512 ? 1 : (512 + tiles - 1) / tiles;
@@ -461,9 +463,9 @@ static int rope_launch(void* qkv, const int* positions, const int* seq_of_token,
   void *qkv, const int *positions, const int *seq_of_token, const float *cos_t,                 \
       const float *sin_t, const int *block_table, void *k_pages, void *v_pages, int n, int H,   \
       int KV, int d, int rot, int table_len, int block_size, int table_stride, int num_blocks,  \
-      int write_kv, int n_seqs, hipStream_t s
+      int write_kv, int n_seqs, int row_len, hipStream_t s
 #define ROPE_ARGS_PACK                                                                           \
-  RopeArgs { H, KV, d, rot, table_len, block_size, table_stride, num_blocks, write_kv, n_seqs }
+  RopeArgs { H, KV, d, rot, table_len, block_size, table_stride, num_blocks, write_kv, n_seqs, row_len }
 KVF_EXPORT int kvf_rope_kvwrite_f32(ROPE_ARGS_DECL) {
   return rope_launch<float>(qkv, positions, seq_of_token, cos_t, sin_t, block_table, k_pages,
                             v_pages, n, ROPE_ARGS_PACK, s);
@@ -471,4 +473,316 @@ KVF_EXPORT int kvf_rope_kvwrite_f32(ROPE_ARGS_DECL) {
 KVF_EXPORT int kvf_rope_kvwrite_bf16(ROPE_ARGS_DECL) {
   return rope_launch<bf16_t>(qkv, positions, seq_of_token, cos_t, sin_t, block_table, k_pages,
                              v_pages, n, ROPE_ARGS_PACK, s);
+}
+
+// ----------------------------------------------------------------------------- learned positions
+// x[n, :] += table[positions[n], :] in fp32 (an absolute position encoding on the embedding
+// output).  A position outside the table adds nothing.
+template <typename T>
+__global__ void add_positions_kernel(float* __restrict__ x, const T* __restrict__ table,
+                                     const int* __restrict__ positions, int h, int table_len) {
+  const int n = blockIdx.x;
+  const int p = positions[n];
+  if (p < 0 || p >= table_len) return;
+  float* o = x + static_cast<size_t>(n) * h;
+  const T* row = table + static_cast<size_t>(p) * h;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) o[i] += Elem<T>::load(row + i);
+}
+template <typename T>
+static int add_positions_launch(float* x, const void* table, const int* positions, int n, int h,
+                                int table_len, hipStream_t s) {
+  if (n <= 0) return 0;
+  hipLaunchKernelGGL(add_positions_kernel<T>, dim3(n), dim3(256), 0, s, x, static_cast<const T*>(table),
+                     positions, h, table_len);
+  return kvf_last_error();
+}
+KVF_EXPORT int kvf_add_positions_f32(float* x, const void* t, const int* p, int n, int h, int len,
+                                     hipStream_t s) { return add_positions_launch<float>(x, t, p, n, h, len, s); }
+KVF_EXPORT int kvf_add_positions_bf16(float* x, const void* t, const int* p, int n, int h, int len,
+                                      hipStream_t s) { return add_positions_launch<bf16_t>(x, t, p, n, h, len, s); }
+
+// ----------------------------------------------------------------------------- norm + token shift
+// For token t of the flat batch, with y(r) = x[r] * rsqrt(mean(x[r]^2) + eps) * w (all fp32):
+//   plain[t]   = y(t)
+//   shifted[t] = y(t) + (prev - y(t)) * mu,   prev = the y of the token before t in its sequence:
+//     zeros at position 0; y(t - 1) where t - 1 belongs to the same query run (computed again
+//     here, with the same order of sums, so that it is the number the other workgroup stores);
+//     state[slot of the sequence] for the first token of a run that continues a sequence.
+// The workgroup of a run's first token is also the one that leaves the y of the run's *last*
+// token in the sequence's state slot, after it has read the slot: no other workgroup touches
+// that slot, so reading and writing it need no order between workgroups.  A sequence without a
+// slot (negative: the padding of a captured batch) has no state.
+template <typename T>
+__global__ __launch_bounds__(256) void norm_shift_kernel(
+    const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ mu,
+    float* __restrict__ state, const int* __restrict__ slot_ids, const int* __restrict__ seq_of_token,
+    const int* __restrict__ cu_q, const int* __restrict__ positions, T* __restrict__ plain,
+    T* __restrict__ shifted, float eps, int h, int n_seqs, int n_slots, int n_tokens) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  int seq = seq_of_token[t];
+  if (seq < 0 || seq >= n_seqs) seq = -1;
+  const int q_first = seq >= 0 ? cu_q[seq] : t;
+  int q_last = seq >= 0 ? cu_q[seq + 1] - 1 : t;
+  if (q_last < t || q_last >= n_tokens) q_last = t;
+  const bool first = t == q_first;
+  const int pos = positions[t];
+  int slot = seq >= 0 ? slot_ids[seq] : -1;
+  if (slot >= n_slots) slot = -1;
+  const float* xr = x + static_cast<size_t>(t) * h;
+  const float inv_h = 1.f / static_cast<float>(h);
+
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
+  const float r = rsqrtf(block_sum(ss, scratch) * inv_h + eps);
+
+  // where the predecessor comes from: 0 nothing, 1 the row before, 2 the state slot
+  const int from = pos <= 0 ? 0 : (!first ? 1 : (slot >= 0 ? 2 : 0));
+  float rp = 0.f;
+  const float* xp = xr - h;
+  if (from == 1) {
+    float sp = 0.f;
+    for (int i = threadIdx.x; i < h; i += blockDim.x) sp = fmaf(xp[i], xp[i], sp);
+    rp = rsqrtf(block_sum(sp, scratch) * inv_h + eps);
+  }
+  const float* st = slot >= 0 ? state + static_cast<size_t>(slot) * h : nullptr;
+  T* po = plain + static_cast<size_t>(t) * h;
+  T* so = shifted + static_cast<size_t>(t) * h;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) {
+    const float y = xr[i] * r * w[i];
+    const float prev = from == 1 ? xp[i] * rp * w[i] : (from == 2 ? st[i] : 0.f);
+    Elem<T>::store(po + i, y);
+    Elem<T>::store(so + i, fmaf(prev - y, mu[i], y));
+  }
+  if (!first || slot < 0) return;
+  // every thread has read the elements of the slot that it is about to write
+  float* sw = state + static_cast<size_t>(slot) * h;
+  if (q_last == t) {
+    for (int i = threadIdx.x; i < h; i += blockDim.x) sw[i] = xr[i] * r * w[i];
+    return;
+  }
+  const float* xl = x + static_cast<size_t>(q_last) * h;
+  float sl = 0.f;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) sl = fmaf(xl[i], xl[i], sl);
+  const float rl = rsqrtf(block_sum(sl, scratch) * inv_h + eps);
+  for (int i = threadIdx.x; i < h; i += blockDim.x) sw[i] = xl[i] * rl * w[i];
+}
+template <typename T>
+static int norm_shift_launch(const float* x, const float* w, const float* mu, float* state,
+                             const int* slot_ids, const int* seq_of_token, const int* cu_q,
+                             const int* positions, void* plain, void* shifted, float eps, int n, int h,
+                             int n_seqs, int n_slots, hipStream_t s) {
+  if (n <= 0) return 0;
+  // one block size for every call: the order of a row's sum of squares must not depend on the batch
+  hipLaunchKernelGGL(norm_shift_kernel<T>, dim3(n), dim3(256), 0, s, x, w, mu, state, slot_ids,
+                     seq_of_token, cu_q, positions, static_cast<T*>(plain), static_cast<T*>(shifted), eps,
+                     h, n_seqs, n_slots, n);
+  return kvf_last_error();
+}
+#define NORM_SHIFT_DECL                                                                          \
+  const float *x, const float *w, const float *mu, float *state, const int *slot_ids,           \
+      const int *seq_of_token, const int *cu_q, const int *positions, void *plain, void *shifted, \
+      float eps, int n, int h, int n_seqs, int n_slots, hipStream_t s
+KVF_EXPORT int kvf_norm_shift_f32(NORM_SHIFT_DECL) {
+  return norm_shift_launch<float>(x, w, mu, state, slot_ids, seq_of_token, cu_q, positions, plain,
+                                  shifted, eps, n, h, n_seqs, n_slots, s);
+}
+KVF_EXPORT int kvf_norm_shift_bf16(NORM_SHIFT_DECL) {
+  return norm_shift_launch<bf16_t>(x, w, mu, state, slot_ids, seq_of_token, cu_q, positions, plain,
+                                   shifted, eps, n, h, n_seqs, n_slots, s);
+}
+
+// ----------------------------------------------------------------------------- gated activations
+// out[m, i] = act(gate_i + bg[i]) * (up_i + bu[i]) in fp32; the input row holds gate at 2i and
+// up at 2i + 1 (`paired`) or gate at i and up at I + i.  act: 0 silu, 1 the tanh form of gelu.
+// The biases are fp32 vectors and may be null.
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  const float u = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+  return 0.5f * z * (1.f + tanhf(u));
+}
+__device__ __forceinline__ float act_f(int act, float z) {
+  return act == 1 ? gelu_tanh_f(z) : z / (1.f + expf(-z));
+}
+template <typename T>
+__global__ void gated_act_kernel(const T* __restrict__ gu, const float* __restrict__ bg,
+                                 const float* __restrict__ bu, T* __restrict__ out, int inter,
+                                 size_t total, int paired, int act) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t m = idx / inter;
+  const int i = static_cast<int>(idx - m * inter);
+  const T* row = gu + m * 2 * static_cast<size_t>(inter);
+  float g = Elem<T>::load(paired ? row + 2 * i : row + i);
+  float u = Elem<T>::load(paired ? row + 2 * i + 1 : row + inter + i);
+  if (bg) g += bg[i];
+  if (bu) u += bu[i];
+  Elem<T>::store(out + idx, act_f(act, g) * u);
+}
+template <typename T>
+static int gated_act_launch(const void* gu, const float* bg, const float* bu, void* out, int m,
+                            int inter, int paired, int act, hipStream_t s) {
+  const size_t total = static_cast<size_t>(m) * inter;
+  if (total == 0) return 0;
+  hipLaunchKernelGGL(gated_act_kernel<T>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, s,
+                     static_cast<const T*>(gu), bg, bu, static_cast<T*>(out), inter, total, paired, act);
+  return kvf_last_error();
+}
+KVF_EXPORT int kvf_gated_act_f32(const void* gu, const float* bg, const float* bu, void* out, int m,
+                                 int inter, int paired, int act, hipStream_t s) {
+  return gated_act_launch<float>(gu, bg, bu, out, m, inter, paired, act, s);
+}
+KVF_EXPORT int kvf_gated_act_bf16(const void* gu, const float* bg, const float* bu, void* out, int m,
+                                  int inter, int paired, int act, hipStream_t s) {
+  return gated_act_launch<bf16_t>(gu, bg, bu, out, m, inter, paired, act, s);
+}
+
+// ----------------------------------------------------------------------------- sigmoid gate
+// y[m, c] *= sigmoid(g[m, c]) for c < cols; rows of y and g are y_stride / g_stride apart.
+template <typename T>
+__global__ void sigmoid_gate_kernel(T* __restrict__ y, const T* __restrict__ g, int cols, int y_stride,
+                                    int g_stride, size_t total) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t m = idx / cols;
+  const int c = static_cast<int>(idx - m * cols);
+  T* yp = y + m * y_stride + c;
+  const float z = Elem<T>::load(g + m * g_stride + c);
+  Elem<T>::store(yp, Elem<T>::load(yp) / (1.f + expf(-z)));
+}
+template <typename T>
+static int sigmoid_gate_launch(void* y, const void* g, int m, int cols, int y_stride, int g_stride,
+                               hipStream_t s) {
+  const size_t total = static_cast<size_t>(m) * cols;
+  if (total == 0) return 0;
+  hipLaunchKernelGGL(sigmoid_gate_kernel<T>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                     s, static_cast<T*>(y), static_cast<const T*>(g), cols, y_stride, g_stride, total);
+  return kvf_last_error();
+}
+KVF_EXPORT int kvf_sigmoid_gate_f32(void* y, const void* g, int m, int cols, int ys, int gs, hipStream_t s) {
+  return sigmoid_gate_launch<float>(y, g, m, cols, ys, gs, s);
+}
+KVF_EXPORT int kvf_sigmoid_gate_bf16(void* y, const void* g, int m, int cols, int ys, int gs, hipStream_t s) {
+  return sigmoid_gate_launch<bf16_t>(y, g, m, cols, ys, gs, s);
+}
+
+// ----------------------------------------------------------------------------- bias on the stream
+// x[m, :] += bias (fp32) for every row.
+__global__ void add_bias_kernel(float* __restrict__ x, const float* __restrict__ bias, int h, size_t total) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < total) x[i] += bias[i % h];
+}
+KVF_EXPORT int kvf_add_bias(float* x, const float* bias, int m, int h, hipStream_t s) {
+  const size_t total = static_cast<size_t>(m) * h;
+  if (total == 0) return 0;
+  hipLaunchKernelGGL(add_bias_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, s, x,
+                     bias, h, total);
+  return kvf_last_error();
+}
+
+// ----------------------------------------------------------------------------- per-layer token input
+// For every token row m of the fp32 stream x (first brought up to date: x[m] += bias, += owed[m],
+// either may be null), with e = side[token[m], col0 .. col0 + dim):
+//   a = gate x[m]                      gate  [dim, h]
+//   g = gelu_tanh(a) * e
+//   y = proj g                         proj  [h, dim]
+//   x[m] += y * rsqrt(mean(y^2) + eps) * w
+// all sums in fp32.  One workgroup per row: the row and g live in LDS; a wave takes every
+// fourth row of `gate` with its lanes side by side along h, a thread takes elements of y with
+// a row of `proj` to itself.  A token id outside the table adds nothing but bias and owed.
+template <typename T, typename D>
+__global__ __launch_bounds__(256) void token_side_kernel(
+    float* __restrict__ x, const float* __restrict__ bias, const D* __restrict__ owed,
+    const int* __restrict__ tokens, const T* __restrict__ side, const T* __restrict__ gate,
+    const T* __restrict__ proj, const float* __restrict__ w, float eps, int h, int dim, int vocab,
+    int side_stride, int col0) {
+  extern __shared__ float side_lds[];  // [h] the row, [dim] g
+  __shared__ float scratch[16];
+  float* row = side_lds;
+  float* g = side_lds + h;
+  const int m = blockIdx.x;
+  const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE, waves = blockDim.x / KVF_WAVE;
+  float* xr = x + static_cast<size_t>(m) * h;
+  const D* orow = owed ? owed + static_cast<size_t>(m) * h : nullptr;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) {
+    float v = xr[i];
+    if (bias) v += bias[i];
+    if (orow) v += Elem<D>::load(orow + i);
+    row[i] = v;
+  }
+  __syncthreads();
+  const int tok = tokens[m];
+  const bool known = tok >= 0 && tok < vocab;
+  const T* e = side + static_cast<size_t>(known ? tok : 0) * side_stride + col0;
+  for (int j = wave; j < dim; j += waves) {
+    const T* gr = gate + static_cast<size_t>(j) * h;
+    float a = 0.f;
+    for (int i = lane; i < h; i += KVF_WAVE) a = fmaf(Elem<T>::load(gr + i), row[i], a);
+    a = wave_sum(a);
+    if (lane == 0) g[j] = known ? gelu_tanh_f(a) * Elem<T>::load(e + j) : 0.f;
+  }
+  __syncthreads();
+  // y stays in registers where the row is short enough, otherwise it is computed twice
+  constexpr int KEEP = 8;
+  float y[KEEP];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < KEEP; ++k) {
+    const int i = threadIdx.x + k * blockDim.x;
+    y[k] = 0.f;
+    if (i < h) {
+      const T* pr = proj + static_cast<size_t>(i) * dim;
+      float acc = 0.f;
+      for (int j = 0; j < dim; ++j) acc = fmaf(Elem<T>::load(pr + j), g[j], acc);
+      y[k] = acc;
+      ss = fmaf(acc, acc, ss);
+    }
+  }
+  for (int i = threadIdx.x + KEEP * blockDim.x; i < h; i += blockDim.x) {
+    const T* pr = proj + static_cast<size_t>(i) * dim;
+    float acc = 0.f;
+    for (int j = 0; j < dim; ++j) acc = fmaf(Elem<T>::load(pr + j), g[j], acc);
+    ss = fmaf(acc, acc, ss);
+  }
+  const float r = rsqrtf(block_sum(ss, scratch) / static_cast<float>(h) + eps);
+#pragma unroll
+  for (int k = 0; k < KEEP; ++k) {
+    const int i = threadIdx.x + k * blockDim.x;
+    if (i < h) xr[i] = fmaf(y[k] * r, w[i], row[i]);
+  }
+  for (int i = threadIdx.x + KEEP * blockDim.x; i < h; i += blockDim.x) {
+    const T* pr = proj + static_cast<size_t>(i) * dim;
+    float acc = 0.f;
+    for (int j = 0; j < dim; ++j) acc = fmaf(Elem<T>::load(pr + j), g[j], acc);
+    xr[i] = fmaf(acc * r, w[i], row[i]);
+  }
+}
+template <typename T, typename D>
+static int token_side_launch(float* x, const float* bias, const void* owed, const int* tokens,
+                             const void* side, const void* gate, const void* proj, const float* w,
+                             float eps, int n, int h, int dim, int vocab, int side_stride, int col0,
+                             hipStream_t s) {
+  if (n <= 0) return 0;
+  const size_t lds = static_cast<size_t>(h + dim) * sizeof(float);
+  if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL((token_side_kernel<T, D>), dim3(n), dim3(256), lds, s, x, bias,
+                     static_cast<const D*>(owed), tokens, static_cast<const T*>(side),
+                     static_cast<const T*>(gate), static_cast<const T*>(proj), w, eps, h, dim, vocab,
+                     side_stride, col0);
+  return kvf_last_error();
+}
+#define TOKEN_SIDE_DECL                                                                          \
+  float *x, const float *bias, const void *owed, int owed_f32, const int *tokens,               \
+      const void *side, const void *gate, const void *proj, const float *w, float eps, int n,   \
+      int h, int dim, int vocab, int side_stride, int col0, hipStream_t s
+KVF_EXPORT int kvf_token_side_f32(TOKEN_SIDE_DECL) {
+  (void)owed_f32;
+  return token_side_launch<float, float>(x, bias, owed, tokens, side, gate, proj, w, eps, n, h, dim,
+                                         vocab, side_stride, col0, s);
+}
+KVF_EXPORT int kvf_token_side_bf16(TOKEN_SIDE_DECL) {
+  if (owed_f32)
+    return token_side_launch<bf16_t, float>(x, bias, owed, tokens, side, gate, proj, w, eps, n, h, dim,
+                                            vocab, side_stride, col0, s);
+  return token_side_launch<bf16_t, bf16_t>(x, bias, owed, tokens, side, gate, proj, w, eps, n, h, dim,
+                                           vocab, side_stride, col0, s);
 }

@@ -154,6 +154,134 @@ def add_rows(x: torch.Tensor, delta: torch.Tensor) -> None:
     _ok(f(x.data_ptr(), delta.data_ptr(), x.shape[0], x.shape[1], _stream()), "add_rows")
 
 
+def add_positions(x: torch.Tensor, table: torch.Tensor, positions: torch.Tensor) -> None:
+    """``x[n] += table[positions[n]]`` for the fp32 stream ``x``: a learned vector per position."""
+    _check(x, "x", F32, (None, None))
+    n, h = x.shape
+    _check(table, "table", None, (None, h))
+    _check(positions, "positions", I32, (None,))
+    if positions.shape[0] < n:
+        raise KernelError("add_positions: positions shorter than the batch")
+    f = _fn("elementwise", f"kvf_add_positions_{_suffix(table.dtype)}",
+            [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p])
+    _ok(f(x.data_ptr(), table.data_ptr(), positions.data_ptr(), n, h, table.shape[0], _stream()),
+        "add_positions")
+
+
+def norm_shift(x: torch.Tensor, weight: torch.Tensor, mu: torch.Tensor, state: torch.Tensor,
+               slot_ids: torch.Tensor, seq_of_token: torch.Tensor, cu_q: torch.Tensor,
+               positions: torch.Tensor, eps: float, plain: torch.Tensor, shifted: torch.Tensor) -> None:
+    """RMS norm and token shift of the fp32 stream in one kernel.  With ``y = norm(x) * weight``:
+    ``plain = y`` and ``shifted[t] = y[t] + (y[t-1] - y[t]) * mu``, where the token before the
+    first one of a query run is read from the sequence's row of ``state`` (zeros at position 0)
+    and the run's last ``y`` is left there.  ``weight``, ``mu``: fp32 ``[h]``; ``state``: fp32
+    ``[slots, h]``; ``slot_ids``: a slot per sequence, negative for none."""
+    _check(x, "x", F32, (None, None))
+    n, h = x.shape
+    _check(weight, "weight", F32, (h,))
+    _check(mu, "mu", F32, (h,))
+    _check(state, "state", F32, (None, h))
+    for t, name in ((slot_ids, "slot_ids"), (seq_of_token, "seq_of_token"), (cu_q, "cu_q"),
+                    (positions, "positions")):
+        _check(t, name, I32, (None,))
+    n_seqs = slot_ids.shape[0]
+    if cu_q.shape[0] < n_seqs + 1 or seq_of_token.shape[0] < n or positions.shape[0] < n:
+        raise KernelError("norm_shift: batch fields shorter than the batch")
+    _check(plain, "plain", None, (n, h))
+    _check(shifted, "shifted", plain.dtype, (n, h))
+    f = _fn("elementwise", f"kvf_norm_shift_{_suffix(plain.dtype)}",
+            [c_void_p] * 10 + [c_float] + [c_int] * 4 + [c_void_p])
+    _ok(f(x.data_ptr(), weight.data_ptr(), mu.data_ptr(), state.data_ptr(), slot_ids.data_ptr(),
+          seq_of_token.data_ptr(), cu_q.data_ptr(), positions.data_ptr(), plain.data_ptr(),
+          shifted.data_ptr(), float(eps), n, h, n_seqs, state.shape[0], _stream()), "norm_shift")
+
+
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def gated_act(gate_up: torch.Tensor, out: torch.Tensor, activation: str, paired: bool = False,
+              gate_bias: torch.Tensor | None = None, up_bias: torch.Tensor | None = None) -> None:
+    """``out[:, i] = act(gate_i + gate_bias[i]) * (up_i + up_bias[i])``; the input row holds gate
+    at ``i`` and up at ``I + i``, or with ``paired`` at ``2i`` and ``2i + 1``.  ``activation``:
+    ``"silu"`` or ``"gelu_tanh"``; the biases are fp32 ``[I]`` or ``None``."""
+    m, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelError("gated_act: input width must be even")
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"gated_act: unknown activation {activation!r}; known: {sorted(ACTIVATIONS)}")
+    _check(gate_up, "gate_up", None, (m, two_i))
+    _check(out, "out", gate_up.dtype, (m, two_i // 2))
+    for b, name in ((gate_bias, "gate_bias"), (up_bias, "up_bias")):
+        if b is not None:
+            _check(b, name, F32, (two_i // 2,))
+    f = _fn("elementwise", f"kvf_gated_act_{_suffix(out.dtype)}",
+            [c_void_p] * 4 + [c_int] * 4 + [c_void_p])
+    _ok(f(gate_up.data_ptr(), gate_bias.data_ptr() if gate_bias is not None else None,
+          up_bias.data_ptr() if up_bias is not None else None, out.data_ptr(), m, two_i // 2,
+          1 if paired else 0, ACTIVATIONS[activation], _stream()), "gated_act")
+
+
+def sigmoid_gate(y: torch.Tensor, gate: torch.Tensor) -> None:
+    """``y *= sigmoid(gate)`` element by element; both ``[M, C]`` with dense rows (row strides may
+    exceed C, so ``gate`` can be a block of columns of a wider product)."""
+    m, c = y.shape
+    _check(y, "y", None, (m, c), contiguous=False)
+    _check(gate, "gate", y.dtype, (m, c), contiguous=False)
+    if y.stride(1) != 1 or gate.stride(1) != 1:
+        raise KernelError("sigmoid_gate: rows must be dense")
+    f = _fn("elementwise", f"kvf_sigmoid_gate_{_suffix(y.dtype)}", [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p])
+    _ok(f(y.data_ptr(), gate.data_ptr(), m, c, y.stride(0) if m > 1 else c,
+          gate.stride(0) if m > 1 else c, _stream()), "sigmoid_gate")
+
+
+def add_bias(x: torch.Tensor, bias: torch.Tensor) -> None:
+    """``x[m] += bias`` for every row of the fp32 stream."""
+    _check(x, "x", F32, (None, None))
+    _check(bias, "bias", F32, (x.shape[1],))
+    f = _fn("elementwise", "kvf_add_bias", [c_void_p, c_void_p, c_int, c_int, c_void_p])
+    _ok(f(x.data_ptr(), bias.data_ptr(), x.shape[0], x.shape[1], _stream()), "add_bias")
+
+
+TOKEN_SIDE_MAX_FLOATS = 16 * 1024   # the row and the gated vector live in 64 KB of LDS
+
+
+def token_side(x: torch.Tensor, tokens: torch.Tensor, side: torch.Tensor, col0: int,
+               gate: torch.Tensor, proj: torch.Tensor, weight: torch.Tensor, eps: float,
+               bias: torch.Tensor | None = None, owed: torch.Tensor | None = None) -> None:
+    """A per-token input into the fp32 stream: with ``e = side[token, col0 : col0 + dim]``,
+    ``y = proj @ (gelu_tanh(gate @ x[m]) * e)`` and ``x[m] += y * rsqrt(mean(y^2) + eps) * weight``.
+    ``bias`` (fp32 ``[h]``) and ``owed`` (``[M, h]``, a product still owed to the stream) are added
+    to ``x[m]`` first and stay in it.  ``gate [dim, h]``, ``proj [h, dim]`` and ``side`` share a
+    type; ``weight`` is fp32."""
+    _check(x, "x", F32, (None, None))
+    n, h = x.shape
+    _check(tokens, "tokens", I32, (None,))
+    if tokens.shape[0] < n:
+        raise KernelError("token_side: token ids shorter than the batch")
+    _check(gate, "gate", None, (None, h))
+    dim = gate.shape[0]
+    _check(proj, "proj", gate.dtype, (h, dim))
+    _check(side, "side", gate.dtype, (None, None))
+    if not 0 <= col0 <= side.shape[1] - dim:
+        raise KernelError(f"token_side: columns {col0}..{col0 + dim} outside the table's {side.shape[1]}")
+    _check(weight, "weight", F32, (h,))
+    if h + dim > TOKEN_SIDE_MAX_FLOATS:
+        raise KernelError(f"token_side: a row of {h} + {dim} floats does not fit the kernel's LDS")
+    if bias is not None:
+        _check(bias, "bias", F32, (h,))
+    if owed is not None:
+        _check(owed, "owed", None, (n, h))
+        if owed.dtype not in (F32, gate.dtype):
+            raise KernelError(f"token_side: owed must be float32 or {gate.dtype}, got {owed.dtype}")
+    f = _fn("elementwise", f"kvf_token_side_{_suffix(gate.dtype)}",
+            [c_void_p, c_void_p, c_void_p, c_int] + [c_void_p] * 5 + [c_float] + [c_int] * 6 + [c_void_p])
+    _ok(f(x.data_ptr(), bias.data_ptr() if bias is not None else None,
+          owed.data_ptr() if owed is not None else None,
+          1 if owed is not None and owed.dtype == F32 else 0, tokens.data_ptr(), side.data_ptr(),
+          gate.data_ptr(), proj.data_ptr(), weight.data_ptr(), float(eps), n, h, dim, side.shape[0],
+          side.shape[1], int(col0), _stream()), "token_side")
+
+
 # ------------------------------------------------------------------------------ SwiGLU gate
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, paired: bool = False) -> None:
     """``out[:, i] = silu(gate_i) * up_i`` where the input row holds gate at ``i`` and up at
@@ -194,10 +322,14 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
     and v into the pages named by the token's sequence row of ``block_table``.  Rotary pairs
     are neighbouring elements ``(2i, 2i + 1)`` of a head; without tables (``None``) q and k stay
     as they are and only the cache is written.  ``k_pages``:
-    ``[num_blocks, KV, block_size, d]``; ``v_pages`` transposed: ``[num_blocks, KV, d, block_size]``."""
+    ``[num_blocks, KV, block_size, d]``; ``v_pages`` transposed: ``[num_blocks, KV, d, block_size]``.
+    A row of ``qkv`` may hold further columns behind q, k and v (what else the same product made);
+    they are left alone."""
     n = qkv.shape[0]
     H, KV, d = num_heads, num_kv_heads, head_dim
-    _check(qkv, "qkv", None, (n, (H + 2 * KV) * d))
+    _check(qkv, "qkv", None, (n, None))
+    if qkv.shape[1] < (H + (2 * KV if write_kv else 0)) * d:
+        raise KernelError(f"rope_kvwrite: rows of {qkv.shape[1]} elements do not hold q, k and v")
     _check(positions, "positions", I32, (None,))
     _check(seq_of_token, "seq_of_token", I32, (None,))
     if positions.shape[0] < n or seq_of_token.shape[0] < n:
@@ -209,10 +341,11 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
     nb, _, bs, _ = k_pages.shape
     _check(v_pages, "v_pages", qkv.dtype, (nb, KV, d, bs))
     f = _fn("elementwise", f"kvf_rope_kvwrite_{_suffix(qkv.dtype)}",
-            [c_void_p] * 8 + [c_int] * 11 + [c_void_p])
+            [c_void_p] * 8 + [c_int] * 12 + [c_void_p])
     _ok(f(qkv.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), cos_p,
           sin_p, block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
-          n, H, KV, d, rot, table_len, bs, stride, nb, 1 if write_kv else 0, n_seqs, _stream()),
+          n, H, KV, d, rot, table_len, bs, stride, nb, 1 if write_kv else 0, n_seqs,
+          qkv.shape[1], _stream()),
         "rope_kvwrite")
 
 
@@ -655,6 +788,14 @@ def _slopes_ptr(slopes, H: int, like: torch.Tensor):
     return slopes.data_ptr()
 
 
+def _keep_first(window: int, keep_first: int) -> int:
+    """Keys kept visible behind a window; without a window every key is visible anyway."""
+    keep = int(keep_first)
+    if keep < 0:
+        raise KernelError(f"attention: keep_first must not be negative, got {keep}")
+    return keep if int(window) > 0 else 0
+
+
 def attention_on_matrix_cores(dtype: torch.dtype, block_size: int) -> bool:
     """The MFMA attention kernels take bf16 and pages of a multiple of 8 tokens; everything else
     (the true 32-bit path above all) runs the vector-ALU kernel."""
@@ -690,27 +831,30 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  block_table: torch.Tensor, cu_q: torch.Tensor, ctx_lens: torch.Tensor,
                  work: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
                  head_dim: int, scale: float, window: int = 0,
-                 slopes: torch.Tensor | None = None, rows_per_item: int | None = None) -> None:
+                 slopes: torch.Tensor | None = None, rows_per_item: int | None = None,
+                 keep_first: int = 0) -> None:
     """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 3]`` rows
     (sequence row, item, item or -1) where a sequence has ``query_len * H/KV`` rows per kv head,
     an item covers ``rows_per_item`` of them (what ``prefill_rows_per_item`` gave when the rows
     were made; by default its answer for one row tile), and the items of one row are taken by
     one workgroup in turn; rows start in the order given (the longest walks first).  ``v_pages`` are transposed:
     ``[num_blocks, KV, head_dim, block_size]``.  ``slopes``: fp32 ``[H]``; the score of key ``j``
-    for a query at position ``p`` of head ``h`` then is ``scale * q.k + slopes[h] * (j - p)``."""
+    for a query at position ``p`` of head ``h`` then is ``scale * q.k + slopes[h] * (j - p)``.
+    ``keep_first``: with a window, the first so many keys of a sequence stay visible behind it."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     _check(work, "work", I32, (None, 3))
+    keep = _keep_first(window, keep_first)
     sl = _slopes_ptr(slopes, H, q)
     nb, _, bs, _ = k_pages.shape
     if rows_per_item is None:
         rows_per_item = prefill_rows_per_item(q.dtype, d, bs)
     if attention_on_matrix_cores(q.dtype, bs):
         f = _fn("attn_mfma", "kvf_attn_mfma_prefill",
-                [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 10 + [c_float, c_void_p, c_void_p])
+                [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 11 + [c_float, c_void_p, c_void_p])
         _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
               cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(), work.shape[0], int(rows_per_item), out.data_ptr(),
-              H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window),
+              H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window), keep,
               n_seqs, float(scale), sl, _stream()), "attn_mfma_prefill")
         return
     if rows_per_item != prefill_rows_per_item(q.dtype, d, bs):
@@ -719,12 +863,12 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     if q.stride(0) % 4 or out.stride(0) % 4:
         raise KernelError("attn_prefill: rows of q and out must start on 16 bytes")
     f = _fn("attn_generic", "kvf_attn_generic",
-            [c_int] + [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 10
+            [c_int] + [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 11
             + [c_float, c_void_p, c_void_p])
     _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
           block_table.data_ptr(), cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(),
           work.shape[0], out.data_ptr(), H, KV, d, bs, nb, block_table.shape[1], q.stride(0),
-          out.stride(0), int(window), n_seqs, float(scale), sl, _stream()), "attn_generic")
+          out.stride(0), int(window), keep, n_seqs, float(scale), sl, _stream()), "attn_generic")
 
 
 def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
@@ -732,17 +876,19 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                 cu_q: torch.Tensor, ctx_lens: torch.Tensor, out: torch.Tensor, num_heads: int,
                 num_kv_heads: int, head_dim: int, scale: float, window: int = 0, splits: int = 1,
                 workspace: tuple[torch.Tensor, torch.Tensor] | None = None,
-                token_is_seq: bool = False, slopes: torch.Tensor | None = None) -> None:
+                token_is_seq: bool = False, slopes: torch.Tensor | None = None,
+                keep_first: int = 0) -> None:
     """Attention of one-token queries: sequence rows ``seq_ids[:num_seqs]`` (or ``0..num_seqs-1``)
     each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys.  The key
     range may be cut into ``splits`` runs; ``workspace`` then holds fp32 partial accumulators
     (``num_seqs * H * splits * d``) and fp32 (max, sum) pairs (``num_seqs * H * splits * 2``).
     ``token_is_seq``: the caller vouches that ``cu_q[i] == i`` for every sequence (a batch of
     single tokens), which spares the matrix-core kernel a dependent load.  ``slopes``: as in
-    ``attn_prefill``."""
+    ``attn_prefill``; ``keep_first`` likewise."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     sl = _slopes_ptr(slopes, H, q)
+    keep = _keep_first(window, keep_first)
     if token_is_seq and seq_ids is not None:
         raise KernelError("attn_decode: token_is_seq is for batches where every sequence decodes")
     if seq_ids is not None:
@@ -765,22 +911,22 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
             raise KernelError("attn_decode: workspace too small")
     if not attention_on_matrix_cores(q.dtype, bs):
         f = _fn("attn_generic", "kvf_attn_generic_decode",
-                [c_int] + [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p, c_void_p])
+                [c_int] + [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p])
         _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
               block_table.data_ptr(), seq_ids.data_ptr() if seq_ids is not None else None,
               None if token_is_seq else cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(),
               pa.data_ptr() if pa is not None else None, pm.data_ptr() if pm is not None else None,
               num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
-              int(window), n_seqs, int(splits), float(scale), sl, _stream()), "attn_generic_decode")
+              int(window), keep, n_seqs, int(splits), float(scale), sl, _stream()), "attn_generic_decode")
         return
     f = _fn("attn_mfma", "kvf_attn_mfma_decode",
-            [c_void_p] * 10 + [c_int] * 12 + [c_float, c_void_p, c_void_p])
+            [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p])
     _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
           seq_ids.data_ptr() if seq_ids is not None else None,
           None if token_is_seq else cu_q.data_ptr(),
           ctx_lens.data_ptr(), out.data_ptr(), pa.data_ptr() if pa is not None else None,
           pm.data_ptr() if pm is not None else None, num_seqs, H, KV, d, bs, nb,
-          block_table.shape[1], q.stride(0), out.stride(0), int(window), n_seqs, int(splits),
+          block_table.shape[1], q.stride(0), out.stride(0), int(window), keep, n_seqs, int(splits),
           float(scale), sl, _stream()), "attn_mfma_decode")
 
 

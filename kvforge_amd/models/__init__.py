@@ -1,1 +1,2 @@
+from kvforge_amd.models import fogorax  # noqa: F401  (registers Fogorax)
 from kvforge_amd.models import llama  # noqa: F401  (registers LlamaForCausalLM)

@@ -35,16 +35,21 @@ class Transformer:
                 raise ValueError(f"call {i} reads the cache of a later call ({c.cache_of})")
             a = spec.blocks[c.layer].mixer.cache_spec
             b = spec.blocks[self.order[c.cache_of].layer].mixer.cache_spec
-            if a != b:
+            if a is None or a.pages != b.pages:
                 raise ValueError(f"call {i} and call {c.cache_of} need different caches: {a} / {b}")
+        # what an owner keeps covers its own window and those of the calls that read its cache
+        kept: dict[int, CacheSpec] = {i: spec.blocks[self.order[i].layer].mixer.cache_spec for i in owners}
+        for i, c in enumerate(self.order):
+            if c.cache_of is not None:
+                kept[c.cache_of] = kept[c.cache_of].covering(spec.blocks[c.layer].mixer.cache_spec)
         by_spec: dict[CacheSpec, list[int]] = {}
         for i in owners:
-            by_spec.setdefault(spec.blocks[self.order[i].layer].mixer.cache_spec, []).append(i)
-        self.cache_groups = [CacheGroup(tuple(ix), cs.pages, cs.window)
+            by_spec.setdefault(kept[i], []).append(i)
+        self.cache_groups = [CacheGroup(tuple(ix), cs.pages, cs.window, cs.keep_first)
                              for cs, ix in by_spec.items()]
         self.state_specs: dict[int, StateSpec] = {
-            i: spec.blocks[c.layer].mixer.state_spec for i, c in enumerate(self.order)
-            if spec.blocks[c.layer].mixer.state_spec is not None}
+            i: spec.blocks[c.layer].state_spec for i, c in enumerate(self.order)
+            if spec.blocks[c.layer].state_spec is not None}
         self.layer_states: list[LayerState] = []
         self._loaded = False
 

@@ -77,55 +77,106 @@ class PagedAttention(Mixer):
     ``rotary``: the rotation of q and k, or ``None`` for none.  ``score_slopes``: one number per
     q head, or ``None``; the score of key ``j`` for a query at position ``p`` of head ``h`` then
     gets ``score_slopes[h] * (j - p)`` added, a position encoding by distance that lives in the
-    scores instead of in q and k."""
+    scores instead of in q and k.
+    ``keep_first``: with a window, the first so many keys of a sequence stay visible behind it
+    (key ``j`` is seen from position ``p`` iff ``j <= p`` and (``p - j < window`` or
+    ``j < keep_first``)), and their pages are kept.
+    ``value_dim``: size of a value head where it differs from the query/key size ``head_dim``.
+    The kernels take one size for both: the heads of the projections are padded with zero rows
+    (zero columns of the output projection) up to the larger of the two, rounded up to the
+    kernels' step of 16, which changes no score and no output.
+    ``gated``: the heads' outputs are multiplied by ``sigmoid(W_g x)`` element by element before
+    the output projection; ``W_g`` reads the same input as the other projections and rides in
+    their product.
+    ``own_kv``: ``False`` for a mixer without key and value projections, which reads the cache
+    of another call (``LayerCall.cache_of``) with queries, mask and gate of its own.
+    ``names``: checkpoint names of the matrices under the prefix, by ``q k v o g``."""
+
+    NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+             "g": "g_proj.weight"}
 
     replayable = True
     settles_residual = True  # its norm kernel adds what is owed to the stream
 
     def __init__(self, prefix: str, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  rotary: RotaryPositions | None, scale: float | None = None,
-                 window: int | None = None, score_slopes=None) -> None:
+                 window: int | None = None, score_slopes=None, keep_first: int = 0,
+                 value_dim: int | None = None, gated: bool = False, own_kv: bool = True,
+                 names: dict[str, str] | None = None) -> None:
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
-        if head_dim % 16 or head_dim > 256:
+        self.dk = int(head_dim)
+        self.dv = int(value_dim) if value_dim is not None else self.dk
+        padded = -(-max(self.dk, self.dv) // 16) * 16
+        if min(self.dk, self.dv) <= 0 or padded > 256:
+            raise ValueError(
+                f"attention kernels take head sizes up to 256, got {self.dk} / {self.dv}")
+        if value_dim is None and head_dim % 16:
             raise ValueError(
                 f"attention kernels take head sizes in steps of 16 up to 256, got {head_dim}")
         self.prefix = prefix
-        self.hidden, self.H, self.KV, self.d = int(hidden), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.hidden, self.H, self.KV, self.d = int(hidden), int(num_heads), int(num_kv_heads), padded
         self.rotary = rotary
-        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.dk)
         self.window = int(window) if window else None
+        self.keep_first = int(keep_first) if self.window else 0
+        if self.keep_first < 0:
+            raise ValueError(f"keep_first must not be negative, got {keep_first}")
+        self.gated, self.own_kv = bool(gated), bool(own_kv)
+        self.names = dict(self.NAMES, **(names or {}))
         self.score_slopes = None if score_slopes is None else [float(v) for v in score_slopes]
         if self.score_slopes is not None and len(self.score_slopes) != self.H:
             raise ValueError(f"score_slopes needs one number per q head ({self.H}), got {len(self.score_slopes)}")
         self.slopes: torch.Tensor | None = None
-        self.cache_spec = CacheSpec(attention_pages(self.KV, self.d), self.window)
+        self.cache_spec = CacheSpec(attention_pages(self.KV, self.d), self.window, self.keep_first)
         self.w_qkv: torch.Tensor | None = None
         self.w_o: torch.Tensor | None = None
 
+    def _matrices(self) -> list[str]:
+        return ["q"] + (["k", "v"] if self.own_kv else []) + (["g"] if self.gated else [])
+
     def weight_specs(self) -> dict[str, WeightSpec]:
-        h, H, KV, d = self.hidden, self.H, self.KV, self.d
-        return {
-            self._name("q_proj.weight"): WeightSpec((H * d, h)),
-            self._name("k_proj.weight"): WeightSpec((KV * d, h)),
-            self._name("v_proj.weight"): WeightSpec((KV * d, h)),
-            self._name("o_proj.weight"): WeightSpec((h, H * d)),
-        }
+        h, H, KV = self.hidden, self.H, self.KV
+        shapes = {"q": (H * self.dk, h), "k": (KV * self.dk, h), "v": (KV * self.dv, h),
+                  "g": (H * self.dv, h)}
+        out = {self._name(self.names[n]): WeightSpec(shapes[n]) for n in self._matrices()}
+        out[self._name(self.names["o"])] = WeightSpec((h, H * self.dv))
+        return out
+
+    def _padded_heads(self, w: torch.Tensor, heads: int, size: int, perm=None) -> torch.Tensor:
+        """Rows of ``heads`` heads of ``size`` rows each, every head padded with zero rows up to
+        the kernels' head size (and its rows permuted first, if asked)."""
+        w = w.view(heads, size, -1)
+        if perm is not None:
+            w = w[:, perm]
+        if size != self.d:
+            w = torch.cat([w, w.new_zeros(heads, self.d - size, w.shape[2])], dim=1)
+        return w.reshape(heads * self.d, -1)
 
     def load(self, tensors: dict[str, torch.Tensor]) -> None:
-        q, k, v = (tensors[self._name(f"{n}_proj.weight")] for n in "qkv")
-        if not (q.dtype == k.dtype == v.dtype):
-            q, k, v = q.float(), k.float(), v.float()
+        mats = {n: tensors[self._name(self.names[n])] for n in self._matrices()}
+        if len({m.dtype for m in mats.values()}) > 1:
+            mats = {n: m.float() for n, m in mats.items()}
         # The kernels rotate neighbouring elements (2i, 2i+1); the checkpoint pairs element i
         # with i + rot/2.  Permuting the rows of the q and k projections inside each head moves
         # the checkpoint's pairs next to each other; q.k does not depend on the order, v and the
         # output projection keep theirs.
         perm = self.pair_permutation()
-        q = q.view(self.H, self.d, -1)[:, perm].reshape(self.H * self.d, -1)
-        k = k.view(self.KV, self.d, -1)[:, perm].reshape(self.KV * self.d, -1)
-        # one product for the three projections: rows of q heads, then k heads, then v heads
-        self.w_qkv = torch.cat([q, k, v], dim=0).contiguous()
-        self.w_o = tensors[self._name("o_proj.weight")]
+        rows = [self._padded_heads(mats["q"], self.H, self.dk, perm)]
+        if self.own_kv:
+            rows += [self._padded_heads(mats["k"], self.KV, self.dk, perm),
+                     self._padded_heads(mats["v"], self.KV, self.dv)]
+        if self.gated:
+            rows.append(self._padded_heads(mats["g"], self.H, self.dv))
+        # one product for all projections: rows of q heads, then k heads, then v heads, then
+        # the gate's heads
+        self.w_qkv = torch.cat(rows, dim=0).contiguous()
+        w_o = tensors[self._name(self.names["o"])]
+        if self.dv != self.d:
+            w_o = torch.cat([w_o.view(self.hidden, self.H, self.dv),
+                             w_o.new_zeros(self.hidden, self.H, self.d - self.dv)], dim=2)
+            w_o = w_o.reshape(self.hidden, self.H * self.d).contiguous()
+        self.w_o = w_o
         self.norm_eps = None
         if self.score_slopes is not None:
             self.slopes = torch.tensor(self.score_slopes, dtype=torch.float32, device=self.w_o.device)
@@ -134,7 +185,7 @@ class PagedAttention(Mixer):
         """``perm[new] = old`` within a head: new elements 2i and 2i+1 are the checkpoint's
         elements i and i + rot/2; elements beyond the rotary width stay."""
         rot = self.rotary.rot_dim if self.rotary is not None else 0
-        perm = torch.arange(self.d)
+        perm = torch.arange(self.dk)
         for i in range(rot // 2):
             perm[2 * i], perm[2 * i + 1] = i, i + rot // 2
         return perm
@@ -149,7 +200,10 @@ class PagedAttention(Mixer):
         (the kernel that fuses the three has no place for it) and keeps its norm a kernel."""
 
     def _hooked(self) -> bool:
-        return type(self).after_projection is not PagedAttention.after_projection
+        """Whether projection, rotation + cache write and attention run as kernels of their
+        own: a variant with a hook between them, a gate, or no keys and values of its own."""
+        return (type(self).after_projection is not PagedAttention.after_projection
+                or self.gated or not self.own_kv)
 
     def absorb_norm(self, norm) -> bool:
         if self._hooked():
@@ -182,7 +236,7 @@ class PagedAttention(Mixer):
         on besides the padded batch size.  A cell is ``KEYS_PER_CUT`` keys of the longest
         context (of the window, for a windowed layer), and the plan is made for the cell's lower
         edge."""
-        ctx = min(shape.max_ctx, self.window) if self.window else shape.max_ctx
+        ctx = min(shape.max_ctx, self.window + self.keep_first) if self.window else shape.max_ctx
         cell = min(ctx // KEYS_PER_CUT, MAX_CUTS)
         return cell, skew_cuts(max(cell * KEYS_PER_CUT, 1), shape.sum_ctx, shape.n)
 
@@ -264,18 +318,21 @@ class PagedAttention(Mixer):
                               layer.k_pages, layer.v_pages, H, KV, d, write_kv=layer.owns_cache,
                               rms_eps=rms, a_owed=owed)
         else:
-            qkv = ws.buf("qkv", (n, (H + 2 * KV) * d), act)
+            qkv = ws.buf("qkv", (n, self.w_qkv.shape[0]), act)
             ops.gemm(x, self.w_qkv, qkv)
             self.after_projection(qkv, step)
-            ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, cos, sin, table,
-                             layer.k_pages, layer.v_pages, H, KV, d, write_kv=layer.owns_cache)
+            if self.own_kv or self.rotary is not None:
+                ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, cos, sin, table,
+                                 layer.k_pages, layer.v_pages, H, KV, d,
+                                 write_kv=layer.owns_cache and self.own_kv)
         out = ws.buf("attn_out", (n, H * d), act)
         window = self.window or 0
         bs = layer.k_pages.shape[2]
         work, rows_per_item = self._prefill_work(step, act, bs)
         if work is not None:
             ops.attn_prefill(qkv, layer.k_pages, layer.v_pages, table, step.cu_q, step.ctx_lens,
-                             work, out, H, KV, d, self.scale, window, self.slopes, rows_per_item)
+                             work, out, H, KV, d, self.scale, window, self.slopes, rows_per_item,
+                             keep_first=self.keep_first)
         if step.n_decode:
             splits = self._decode_cuts(step, ops.attention_on_matrix_cores(act, bs))
             workspace = None
@@ -286,5 +343,8 @@ class PagedAttention(Mixer):
                             step.n_decode, step.cu_q, step.ctx_lens, out, H, KV, d, self.scale,
                             window, splits, workspace,
                             token_is_seq=step.decode_seq_ids is None and work is None,
-                            slopes=self.slopes)
+                            slopes=self.slopes, keep_first=self.keep_first)
+        if self.gated:
+            g0 = (H + (2 * KV if self.own_kv else 0)) * d
+            ops.sigmoid_gate(out, qkv[:, g0:g0 + H * d])
         add_product(step, out, self.w_o, residual, owed=owed)

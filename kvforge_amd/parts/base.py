@@ -70,11 +70,23 @@ class CacheSpec:
     per token, say).
 
     ``window``: ``None`` keeps every position; ``w`` keeps the last ``w`` positions, and pages
-    wholly behind the window are given back while the request is live.  Layers with equal specs
-    form one cache group with pages and block tables of its own."""
+    wholly behind the window are given back while the request is live.  ``keep_first``: with a
+    window, the first so many positions of a sequence are kept as well (their pages are never
+    given back).  Layers with equal specs form one cache group with pages and block tables of
+    its own."""
 
     pages: tuple[PageTensor, ...]
     window: int | None = None
+    keep_first: int = 0
+
+    def covering(self, other: "CacheSpec") -> "CacheSpec":
+        """The spec that keeps what either of two readers of the same pages needs."""
+        if self.pages != other.pages:
+            raise ValueError(f"pages differ: {self.pages} / {other.pages}")
+        if self.window is None or other.window is None:
+            return CacheSpec(self.pages, None, 0)
+        return CacheSpec(self.pages, max(self.window, other.window),
+                         max(self.keep_first, other.keep_first))
 
 
 @dataclass(frozen=True)
@@ -242,6 +254,13 @@ class Block(Part):
 
     mixer: Mixer
 
+    @property
+    def state_spec(self) -> StateSpec | None:
+        """Fixed-size state per live request that a call of this block keeps from step to step
+        (``LayerState.state``): by default whatever its mixer declares.  A block with state of
+        its own (the last token's activations, say) declares it here instead."""
+        return self.mixer.state_spec
+
     def parts(self) -> list[Part]:
         raise NotImplementedError
 
@@ -314,7 +333,8 @@ def add_product(step: "Step", a: torch.Tensor, w: torch.Tensor, residual: torch.
 class LayerCall:
     """One entry of the run order: run block ``layer``.  ``cache_of``: ``None`` gives the call a
     cache of its own, which it writes and reads; an index into the run order (of an earlier
-    call) makes it read that call's cache and write none."""
+    call) makes it read that call's cache and write none.  The two mixers must declare the same
+    page tensors; their windows may differ, and the owner then keeps what either needs."""
 
     layer: int
     cache_of: int | None = None

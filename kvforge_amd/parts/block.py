@@ -4,7 +4,11 @@ mixer's and the feed-forward's last products add into it."""
 
 from __future__ import annotations
 
-from kvforge_amd.parts.base import Block, FeedForward, LayerState, Mixer, Norm, Part
+import torch
+
+from kvforge_amd.kernels import ops
+from kvforge_amd.parts.base import (Block, FeedForward, LayerState, Mixer, Norm, Part, StateSpec,
+                                    WeightSpec)
 from kvforge_amd.registry import register_block
 
 
@@ -41,3 +45,88 @@ class PreNormBlock(Block):
             x = step.ws.buf("normed", tuple(residual.shape), step.act_dtype)
             self.ffn_norm.forward(residual, x, add=step.take_owed(residual))
             self.ffn.forward(x, step, residual)
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """One norm, both sublayers read its output: ``h = norm(x); x += mixer(h) + ffn(h)`` (``ffn``
+    may be ``None``), then an optional part that feeds something more into the stream
+    (``after``, called as ``after.forward(residual, step, bias=...)``).
+
+    ``shift_name``: checkpoint name of a vector ``mu [hidden]``; the *mixer* then reads
+    ``h_t + (h_{t-1} - h_t) * mu`` instead of ``h_t`` (token shift: ``h_{t-1}`` is the previous
+    token's ``h`` before this replacement, zeros for a sequence's first token), while the
+    feed-forward reads ``h`` as it is.  The last ``h`` of every live sequence is the block's
+    state (one fp32 row per request and call), so that a prompt may be cut anywhere.  Norm,
+    shift and the state's upkeep are one kernel."""
+
+    def __init__(self, norm: Norm, mixer: Mixer, ffn: FeedForward | None, hidden: int,
+                 shift_name: str | None = None, after: Part | None = None) -> None:
+        self.norm, self.mixer, self.ffn, self.after = norm, mixer, ffn, after
+        self.hidden, self.shift_name = int(hidden), shift_name
+        self.mu: torch.Tensor | None = None
+        if shift_name is not None:
+            if mixer.state_spec is not None:
+                raise ValueError("token shift beside a mixer with state of its own is not supported")
+            if not hasattr(norm, "weight") or not hasattr(norm, "eps"):
+                raise ValueError("token shift is fused with an RMS norm (a norm with weight and eps)")
+        if ffn is not None and after is not None and hasattr(ffn, "defer_down_bias"):
+            ffn.defer_down_bias = True   # `after` adds it on its way
+
+    @property
+    def state_spec(self) -> StateSpec | None:
+        if self.shift_name is not None:
+            return StateSpec((self.hidden,), torch.float32)
+        return self.mixer.state_spec
+
+    def parts(self) -> list[Part]:
+        return [p for p in (self.norm, self.mixer, self.ffn, self.after) if p is not None]
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        out = super().weight_specs()
+        if self.shift_name is not None:
+            out[self.shift_name] = WeightSpec((self.hidden,), init="normal", std=0.3)
+        return out
+
+    def load(self, tensors) -> None:
+        super().load(tensors)
+        if self.shift_name is not None:
+            self.mu = tensors[self.shift_name].float().contiguous()
+
+    def kernel_modules(self, dtype) -> set[str]:
+        return super().kernel_modules(dtype) | {"elementwise"}
+
+    def held_tensors(self) -> list[torch.Tensor]:
+        return super().held_tensors() + ([self.mu] if self.mu is not None else [])
+
+    def num_bytes(self) -> int:
+        return super().num_bytes() + (4 * self.mu.numel() if self.mu is not None else 0)
+
+    @property
+    def replayable(self) -> bool:
+        return all(p.replayable for p in self.parts())
+
+    def forward(self, residual, step, layer: LayerState) -> None:
+        shape = tuple(residual.shape)
+        h = step.ws.buf("parallel_normed", shape, step.act_dtype)
+        if self.mu is not None:
+            step.settle()
+            hs = step.ws.buf("parallel_shifted", shape, step.act_dtype)
+            w = self.norm.weight
+            if w.dtype != torch.float32:
+                w = self.norm.weight = w.float()
+            ops.norm_shift(residual, w, self.mu, layer.state, step.slot_ids, step.seq_of_token,
+                           step.cu_q, step.positions, self.norm.eps, h, hs)
+        else:
+            self.norm.forward(residual, h, add=step.take_owed(residual))
+            hs = h
+        self.mixer.forward(hs, step, layer, residual)
+        bias = None
+        if self.ffn is not None:
+            if not self.ffn.settles_residual:
+                step.settle()
+            self.ffn.forward(h, step, residual)
+            if getattr(self.ffn, "defer_down_bias", False):
+                bias = self.ffn.down_bias
+        if self.after is not None:
+            self.after.forward(residual, step, bias=bias)

@@ -9,19 +9,21 @@ from kvforge_amd.parts.base import Embedding, Head, WeightSpec
 
 
 class TokenEmbedding(Embedding):
-    """``h0 = table[ids]`` into the fp32 residual stream; no scaling."""
+    """``h0 = table[ids]`` into the fp32 residual stream; no scaling.  ``tensor``: the table's
+    whole checkpoint name where it is not ``<prefix>.weight``."""
 
     replayable = True
 
-    def __init__(self, prefix: str, vocab: int, hidden: int) -> None:
+    def __init__(self, prefix: str, vocab: int, hidden: int, tensor: str | None = None) -> None:
         self.prefix, self.vocab, self.hidden = prefix, int(vocab), int(hidden)
+        self.tensor = tensor if tensor is not None else self._name("weight")
         self.table: torch.Tensor | None = None
 
     def weight_specs(self) -> dict[str, WeightSpec]:
-        return {self._name("weight"): WeightSpec((self.vocab, self.hidden))}
+        return {self.tensor: WeightSpec((self.vocab, self.hidden))}
 
     def load(self, tensors: dict[str, torch.Tensor]) -> None:
-        self.table = tensors[self._name("weight")]
+        self.table = tensors[self.tensor]
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
         return {"elementwise"}
@@ -39,21 +41,22 @@ class TokenEmbedding(Embedding):
 
 class LMHead(Head):
     """``logits = x @ W^T`` in fp32 output.  ``tied_to``: the checkpoint name of the embedding
-    table when the head shares it (then no tensor of its own is expected)."""
+    table when the head shares it (then no tensor of its own is expected).  ``tensor``: the
+    matrix's whole checkpoint name where it is not ``<prefix>.weight``."""
 
     replayable = True
 
-    def __init__(self, prefix: str, vocab: int, hidden: int, tied_to: str | None = None) -> None:
+    def __init__(self, prefix: str, vocab: int, hidden: int, tied_to: str | None = None,
+                 tensor: str | None = None) -> None:
         self.prefix, self.vocab, self.hidden, self.tied_to = prefix, int(vocab), int(hidden), tied_to
+        self.tensor = tied_to if tied_to is not None else (tensor if tensor is not None else self._name("weight"))
         self.weight: torch.Tensor | None = None
 
     def weight_specs(self) -> dict[str, WeightSpec]:
-        if self.tied_to is not None:
-            return {self.tied_to: WeightSpec((self.vocab, self.hidden))}
-        return {self._name("weight"): WeightSpec((self.vocab, self.hidden))}
+        return {self.tensor: WeightSpec((self.vocab, self.hidden))}
 
     def load(self, tensors: dict[str, torch.Tensor]) -> None:
-        self.weight = tensors[self.tied_to if self.tied_to is not None else self._name("weight")]
+        self.weight = tensors[self.tensor]
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
         return {"gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())

@@ -1,4 +1,6 @@
-"""SwiGLU feed-forward: ``down(silu(gate(x)) * up(x))`` (src/tokenvault/model.py:118-132)."""
+"""Gated feed-forward: ``down(act(gate(x)) * up(x))``.  ``SwiGLU`` is the form with ``act = silu``
+and no biases (src/tokenvault/model.py:118-132); ``GatedFeedForward`` takes the activation, biases
+on the three projections and the checkpoint names as arguments."""
 
 from __future__ import annotations
 
@@ -82,3 +84,76 @@ class SwiGLU(FeedForward):
             ops.gemm(x, self.w_gate_up, gu)
             ops.silu_mul(gu, act, paired=True)
         add_product(step, act, self.w_down, residual)
+
+
+@register_feed_forward("gated")
+class GatedFeedForward(SwiGLU):
+    """``down(act(gate x + b_gate) * (up x + b_up)) + b_down``.
+
+    ``activation``: ``"silu"`` or ``"gelu_tanh"`` (``0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))``).
+    ``bias``: whether the three projections have biases; they are held in fp32 and added in
+    fp32, the first two inside the activation kernel.  The bias of the down projection belongs
+    to the stream: ``forward`` adds it with a kernel of its own unless the block asks to add it
+    itself (``defer_down_bias``), in which case it is found in ``down_bias``.
+    ``names``: checkpoint names under the prefix, by ``gate up down``; a bias is ``<name><bias_suffix>``."""
+
+    NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+
+    def __init__(self, prefix: str, hidden: int, intermediate: int, activation: str = "silu",
+                 bias: bool = False, names: dict[str, str] | None = None,
+                 bias_suffix: str = ".bias") -> None:
+        super().__init__(prefix, hidden, intermediate)
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {sorted(ops.ACTIVATIONS)}")
+        self.activation, self.bias = activation, bool(bias)
+        self.names = dict(self.NAMES, **(names or {}))
+        self.bias_suffix = bias_suffix
+        self.gate_bias = self.up_bias = self.down_bias = None
+        self.defer_down_bias = False
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        shapes = {"gate": (self.inter, self.hidden), "up": (self.inter, self.hidden),
+                  "down": (self.hidden, self.inter)}
+        out = {self._name(self.names[n]): WeightSpec(sh) for n, sh in shapes.items()}
+        if self.bias:
+            out.update({self._name(self.names[n] + self.bias_suffix): WeightSpec((sh[0],))
+                        for n, sh in shapes.items()})
+        return out
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        g, u = tensors[self._name(self.names["gate"])], tensors[self._name(self.names["up"])]
+        if g.dtype != u.dtype:
+            g, u = g.float(), u.float()
+        self.w_gate_up = torch.stack([g, u], dim=1).reshape(2 * self.inter, self.hidden).contiguous()
+        self.w_down = tensors[self._name(self.names["down"])]
+        self.norm_eps = None
+        if self.bias:
+            self.gate_bias, self.up_bias, self.down_bias = (
+                tensors[self._name(self.names[n] + self.bias_suffix)].float().contiguous()
+                for n in ("gate", "up", "down"))
+
+    def absorb_norm(self, norm) -> bool:
+        return False
+
+    def num_bytes(self) -> int:
+        return super().num_bytes() + sum(4 * b.numel() for b in (self.gate_bias, self.up_bias, self.down_bias)
+                                         if b is not None)
+
+    def held_tensors(self) -> list[torch.Tensor]:
+        return super().held_tensors() + [b for b in (self.gate_bias, self.up_bias, self.down_bias)
+                                         if b is not None]
+
+    def forward(self, x, step, residual) -> None:
+        """``x``: normalised activations."""
+        n = x.shape[0]
+        ws, dt = step.ws, step.act_dtype
+        step.settle()
+        gu = ws.buf("gate_up", (n, 2 * self.inter), dt)
+        ops.gemm(x, self.w_gate_up, gu)
+        act = ws.buf("ffn_act", (n, self.inter), dt)
+        ops.gated_act(gu, act, self.activation, paired=True, gate_bias=self.gate_bias,
+                      up_bias=self.up_bias)
+        add_product(step, act, self.w_down, residual)
+        if self.down_bias is not None and not self.defer_down_bias:
+            step.settle()
+            ops.add_bias(residual, self.down_bias)

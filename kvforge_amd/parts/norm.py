@@ -43,3 +43,24 @@ class RMSNorm(Norm):
         when it is itself held in bf16 (a weight stored in 32-bit stays a 32-bit multiply)."""
         return (self.weight is not None and self.weight.dtype == torch.bfloat16
                 and matrix.dtype == torch.bfloat16 and matrix.shape[1] == self.width)
+
+
+@register_norm("rmsnorm_scalar")
+class ScalarRMSNorm(RMSNorm):
+    """RMS norm whose gain is one number for all coordinates: ``y = x * rsqrt(mean(x^2) + eps) * g``.
+    The checkpoint holds ``g`` as a tensor without dimensions under ``name``; it is kept as an
+    fp32 vector of ``width`` equal entries, which is what the norm kernels multiply by."""
+
+    def __init__(self, name: str, width: int, eps: float) -> None:
+        super().__init__("", width, eps)
+        self.name = name
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {self.name: WeightSpec((), init="norm", std=0.1)}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        g = tensors[self.name]
+        self.weight = g.float().reshape(1).expand(self.width).contiguous()
+
+    def foldable_into(self, matrix: torch.Tensor) -> bool:
+        return False

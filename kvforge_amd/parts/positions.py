@@ -14,7 +14,7 @@ import math
 import torch
 
 from kvforge_amd.config.model import RopeScaling
-from kvforge_amd.parts.base import Positions
+from kvforge_amd.parts.base import Positions, WeightSpec
 from kvforge_amd.registry import register_positions
 
 
@@ -60,3 +60,33 @@ class RotaryPositions(Positions):
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
         return {"elementwise"}
+
+
+@register_positions("learned")
+class LearnedPositions(Positions):
+    """An absolute encoding: a learned vector per position, ``table[p]``, added to the embedding
+    of the token at position ``p`` as it is (no scale).  ``name``: the table's checkpoint name,
+    ``[max_positions, width]``."""
+
+    replayable = True
+
+    def __init__(self, name: str, max_positions: int, width: int) -> None:
+        self.name, self.max_positions, self.width = name, int(max_positions), int(width)
+        self.table: torch.Tensor | None = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {self.name: WeightSpec((self.max_positions, self.width))}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        self.table = tensors[self.name]
+
+    def kernel_modules(self, dtype: torch.dtype) -> set[str]:
+        return {"elementwise"}
+
+    def held_tensors(self) -> list[torch.Tensor]:
+        return [] if self.table is None else [self.table]
+
+    def on_embedding(self, residual: torch.Tensor, step) -> None:
+        from kvforge_amd.kernels import ops
+
+        ops.add_positions(residual, self.table, step.positions)

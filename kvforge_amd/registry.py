@@ -1,4 +1,4 @@
-"""One registry from an architecture's name (``architectures[0]`` of config.json) to its typed
+"""One registry from an architecture's name (``architectures[0]`` or ``architecture`` of config.json) to its typed
 configuration and the builder that assembles its model from parts; and registries of the parts
 themselves by kind, so a builder can choose a mixer, feed-forward, norm or position encoding
 layer by layer from what the configuration says.
@@ -70,11 +70,20 @@ def get_architecture(name: str) -> Architecture:
             f"architecture {name!r} is not registered; known: {sorted(ARCHITECTURES)}") from None
 
 
-def config_from_dict(d: dict[str, Any]) -> ModelConfig:
+def architecture_name(d: dict[str, Any]) -> str:
+    """The registry key a config.json names: the first of ``architectures`` (a list, as the
+    Hugging Face files write it) or ``architecture`` (one name)."""
     archs = d.get("architectures")
-    if not archs:
-        raise ConfigError("config.json lacks 'architectures'")
-    return get_architecture(archs[0]).config_cls.from_dict(d)
+    if isinstance(archs, (list, tuple)) and archs:
+        return str(archs[0])
+    name = d.get("architecture")
+    if isinstance(name, str) and name:
+        return name
+    raise ConfigError("config.json lacks 'architectures' (or 'architecture')")
+
+
+def config_from_dict(d: dict[str, Any]) -> ModelConfig:
+    return get_architecture(architecture_name(d)).config_cls.from_dict(d)
 
 
 def config_from_folder(folder: str) -> ModelConfig:
