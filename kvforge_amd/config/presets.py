@@ -63,6 +63,31 @@ PRESETS: dict[str, dict[str, Any]] = {
 }
 
 
+def fogorax(vocab: int, width: int, layers: int, heads: int, kv_heads: int, dim: int, ff: int,
+            window: int, keep_first: int, side_dim: int, max_positions: int, vdim: int | None = None,
+            share_every: int = 2, eps: float = 1e-5) -> dict[str, Any]:
+    """A Fogorax config.json of ``layers`` equal layers; of every ``share_every`` layers the first
+    projects keys and values and the others read its cache (1: every layer its own)."""
+    out = []
+    for i in range(layers):
+        mixer: dict[str, Any] = {"dim": dim, "heads": heads, "kv_heads": kv_heads,
+                                 "mask": {"keep_first": keep_first, "size": window},
+                                 "scale": float(dim) ** -0.5, "vdim": vdim if vdim is not None else dim}
+        if share_every > 1 and i % share_every:
+            mixer["kv_from"] = i - i % share_every
+        out.append({"mixer": mixer, "mlp": {"ff": ff, "kind": "dense"}, "type": "attention"})
+    return {"architecture": "Fogorax", "layers": out, "max_positions": max_positions,
+            "norm": {"eps": eps}, "token_side": {"dim": side_dim} if side_dim else None,
+            "vocab": vocab, "width": width}
+
+
+PRESETS["fogorax-tiny"] = fogorax(vocab=300, width=96, layers=4, heads=6, kv_heads=2, dim=16, ff=160,
+                                  window=24, keep_first=2, side_dim=8, max_positions=512, vdim=32)
+# the layer sizes of llama-1b in this design: what its kernels are measured at
+PRESETS["fogorax-1b"] = fogorax(vocab=128256, width=2048, layers=16, heads=32, kv_heads=8, dim=64,
+                                ff=8192, window=1024, keep_first=4, side_dim=64, max_positions=131072)
+
+
 def preset_dict(name: str) -> dict[str, Any]:
     try:
         return dict(PRESETS[name])

@@ -67,8 +67,10 @@ def main(argv: list[str] | None = None) -> int:
     block_size = args.block_size
     num_blocks = pool_pages(args.max_tokens, block_size)
     capacity = num_blocks * block_size
+    # a request may be longer than the pool where windows give pages back while it lives
+    longest = max(capacity, min(int(model.config.max_position_embeddings), 1 << 20))
     runner = ModelRunner(model, block_size, num_blocks, max_num_seqs=args.max_live,
-                         max_num_batched_tokens=capacity, max_model_len=capacity)
+                         max_num_batched_tokens=capacity, max_model_len=longest)
     _say(f"ready: {num_blocks} pages of {block_size} tokens per cache group")
     held: dict[str, int] = {}
     cache = runner.cache

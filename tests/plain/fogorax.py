@@ -22,6 +22,16 @@ import math
 import torch
 
 
+def stored(x: torch.Tensor, store: torch.dtype | None) -> torch.Tensor:
+    """``x`` as it is after a trip through memory in type ``store`` (rounded and widened
+    again), or unchanged for ``None``.  ``forward(..., store=torch.bfloat16)`` rounds so every
+    tensor that an engine serving in bfloat16 may keep in 16 bits between two operations
+    (normalised rows, projections, attention outputs, activations), and nothing else: the
+    stream, norms, scores and softmax stay as they are.  What that run differs from the
+    unrounded one by is the size of rounding alone."""
+    return x if store is None else x.to(store).to(x.dtype)
+
+
 def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
     return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
 
@@ -55,30 +65,36 @@ def window_mask(T: int, size: int, keep_first: int) -> torch.Tensor:
     return (j <= i) & ((i - j < size) | (j < keep_first))
 
 
+def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
+                     mask: torch.Tensor) -> torch.Tensor:
+    """Softmax attention of ``q [Tq, heads, dim]`` over ``k [Tk, kv_heads, dim]`` and
+    ``v [Tk, kv_heads, vdim]``; query head ``h`` uses key/value head ``h // (heads / kv_heads)``;
+    ``mask [Tq, Tk]`` says which keys a query sees.  Returns ``[Tq, heads, vdim]``."""
+    per = q.shape[1] // k.shape[1]
+    out = []
+    for h in range(q.shape[1]):
+        s = (q[:, h] @ k[:, h // per].T) * scale
+        s = s.masked_fill(~mask, float("-inf"))
+        out.append(torch.softmax(s, dim=-1) @ v[:, h // per])
+    return torch.stack(out, dim=1)
+
+
 def gated_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gate: torch.Tensor,
                     heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
                     mask: torch.Tensor) -> torch.Tensor:
     """``q [T, heads*dim]``, ``k [T, kv_heads*dim]``, ``v [T, kv_heads*vdim]``,
     ``gate [T, heads*vdim]`` (before the sigmoid).  Returns the gated heads side by side."""
     T = q.shape[0]
-    per = heads // kv_heads
-    out = []
-    for h in range(heads):
-        g = h // per
-        qh = q[:, h * dim:(h + 1) * dim]
-        kh = k[:, g * dim:(g + 1) * dim]
-        vh = v[:, g * vdim:(g + 1) * vdim]
-        s = (qh @ kh.T) * scale
-        s = s.masked_fill(~mask, float("-inf"))
-        out.append(torch.softmax(s, dim=-1) @ vh)
-    return torch.cat(out, dim=-1) * torch.sigmoid(gate)
+    o = masked_attention(q.view(T, heads, dim), k.view(T, kv_heads, dim), v.view(T, kv_heads, vdim),
+                         scale, mask)
+    return o.reshape(T, heads * vdim) * torch.sigmoid(gate)
 
 
-def dense_ff(h: torch.Tensor, w: dict, p: str) -> torch.Tensor:
+def dense_ff(h: torch.Tensor, w: dict, p: str, store: torch.dtype | None = None) -> torch.Tensor:
     """``down(gelu(gate h + b) * (up h + b)) + b`` with tensors ``p.gate``, ``p.gate.b`` ..."""
-    a = gelu_tanh(h @ w[p + ".gate"].T + w[p + ".gate.b"])
-    b = h @ w[p + ".up"].T + w[p + ".up.b"]
-    return (a * b) @ w[p + ".down"].T + w[p + ".down.b"]
+    a = gelu_tanh(stored(h @ w[p + ".gate"].T, store) + w[p + ".gate.b"])
+    b = stored(h @ w[p + ".up"].T, store) + w[p + ".up.b"]
+    return stored(a * b, store) @ w[p + ".down"].T + w[p + ".down.b"]
 
 
 def token_side(x: torch.Tensor, side_rows: torch.Tensor, gate: torch.Tensor, proj: torch.Tensor,
@@ -90,9 +106,9 @@ def token_side(x: torch.Tensor, side_rows: torch.Tensor, gate: torch.Tensor, pro
 
 
 def forward(config: dict, weights: dict, tokens, dtype: torch.dtype = torch.float32,
-            layers_out: list | None = None) -> torch.Tensor:
+            layers_out: list | None = None, store: torch.dtype | None = None) -> torch.Tensor:
     """Logits ``[T, vocab]`` of one sequence.  ``layers_out``: a list that receives the stream
-    after every layer."""
+    after every layer.  ``store``: see ``stored``."""
     w = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     tok = torch.as_tensor(tokens, dtype=torch.long)
     T = tok.shape[0]
@@ -106,25 +122,39 @@ def forward(config: dict, weights: dict, tokens, dtype: torch.dtype = torch.floa
         m = layer["mixer"]
         p = f"l{i}"
         h = scalar_norm(x, w[p + ".norm1"], eps)
-        hs = token_shift(h, w[p + ".shift"])
+        hs = stored(token_shift(h, w[p + ".shift"]), store)
+        h = stored(h, store)
         H, G, d, dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
         if m.get("kv_from") is not None:
             k, v = kv[int(m["kv_from"])]
         else:
-            k, v = hs @ w[p + ".mix.k"].T, hs @ w[p + ".mix.v"].T
+            k, v = stored(hs @ w[p + ".mix.k"].T, store), stored(hs @ w[p + ".mix.v"].T, store)
             kv[i] = (k, v)
-        heads = gated_attention(hs @ w[p + ".mix.q"].T, k, v, hs @ w[p + ".mix.g"].T, H, G, d, dv,
-                                float(m["scale"]),
-                                window_mask(T, int(m["mask"]["size"]), int(m["mask"]["keep_first"])))
+        mask = window_mask(T, int(m["mask"]["size"]), int(m["mask"]["keep_first"]))
+        q, g = stored(hs @ w[p + ".mix.q"].T, store), stored(hs @ w[p + ".mix.g"].T, store)
+        if store is None:
+            heads = gated_attention(q, k, v, g, H, G, d, dv, float(m["scale"]), mask)
+        else:       # the heads make a trip through memory before the gate
+            heads = stored(gated_attention(q, k, v, torch.full_like(g, float("inf")), H, G, d, dv,
+                                           float(m["scale"]), mask), store)
+            heads = stored(heads * torch.sigmoid(g), store)
         delta = heads @ w[p + ".mix.o"].T
         if layer.get("mlp") is not None:
             if layer["mlp"]["kind"] != "dense":
                 raise ValueError(f"layer {i}: unknown feed-forward {layer['mlp']['kind']!r}")
-            delta = delta + dense_ff(h, w, p + ".mlp")
+            delta = delta + dense_ff(h, w, p + ".mlp", store)
         x = x + delta
         if sdim:
             x = x + token_side(x, w["side.embed"][tok][:, i * sdim:(i + 1) * sdim],
                                w[p + ".side.gate"], w[p + ".side.proj"], w[p + ".side.norm"], eps)
         if layers_out is not None:
             layers_out.append(x.clone())
-    return scalar_norm(x, w["final.norm"], eps) @ w["head"].T
+    return stored(scalar_norm(x, w["final.norm"], eps), store) @ w["head"].T
+
+
+def greedy(config: dict, weights: dict, prompt, n: int, dtype: torch.dtype = torch.float32) -> list[int]:
+    """``n`` tokens after ``prompt``, each the largest logit of the whole sequence so far."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(forward(config, weights, toks, dtype)[-1].argmax()))
+    return toks[len(prompt):]
