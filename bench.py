@@ -5,6 +5,7 @@
                     [--preset llama-1b|llama-3b|llama-8b] [--context-len 8192]
     python bench.py --phase mixed --preset llama-3b --batch 32 --steps 256
     python bench.py --phase burst --preset small [--dtype float32]
+    python bench.py --phase fogorax [--dtype float32] [--steps 64] [--batch 8]
 
 Default run: the layer sizes of Llama 3.2 1B (16 layers, hidden 2048, 32 heads, 8 kv heads, head
 size 64, SwiGLU 8192, vocabulary 128256, llama3 rope scaling, tied embeddings), random weights
@@ -20,6 +21,10 @@ Llama 3.2 3B shape (32 requests, prompts of 128 to 4,096 tokens, chunked prefill
 Llama 3.1 8B shape, all 32 layers (batch 16 at 32,768-token prompts, 128 new tokens; before it
 decode at batch 1 and 8 over 512-token prompts); the 32-bit, 3B and 8B models draw their random
 weights on the device.
+``--phase fogorax`` leaves the default workload alone and measures the Fogorax design instead:
+decode (at ``--batch`` over ``--prompt-len``-token prompts) and a 2,048-token prefill at a few
+layer sizes, each beside a Llama model of equal sizes whose layers all have the same sliding
+window, the engine's closest existing model.
 Peaks are the published MI355X ones: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bf16, 157.3 TFLOP/s
 for fp32.
 """
@@ -371,6 +376,56 @@ def products_run(cfg, rows, repeats=6):
     return out
 
 
+# (name, width, heads, kv heads, head size, feed-forward, layers, vocabulary, per-layer token input)
+FOGORAX_SIZES = [("w1024", 1024, 16, 4, 64, 4096, 8, 32000, 32),
+                 ("w2048", 2048, 32, 8, 64, 8192, 8, 128256, 64),
+                 ("w4096", 4096, 32, 8, 128, 14336, 4, 128256, 128)]
+FOGORAX_WINDOW, FOGORAX_KEEP = 1024, 4
+
+
+def fogorax_points(dtype, batch, prompt_len, steps, warmup, use_graphs=True):
+    """Fogorax at a few sizes that resemble a real model's layers, beside a Llama model of the
+    same sizes with the same sliding window in every layer; random weights drawn on the device.
+    Per size and model: ms per decode step, its share of the HBM roofline, tokens a second of a
+    2,048-token prefill and its share of the matrix-core peak."""
+    import torch
+    from kvforge_amd.config.presets import fogorax as fogorax_config
+
+    elem = 2 if dtype == "bfloat16" else 4
+    out = {}
+    for name, w, H, KV, d, ff, layers, vocab, side in FOGORAX_SIZES:
+        llama = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": vocab,
+                 "hidden_size": w, "num_hidden_layers": layers, "num_attention_heads": H,
+                 "num_key_value_heads": KV, "head_dim": d, "intermediate_size": ff,
+                 "max_position_embeddings": CONTEXT_CAP, "rope_theta": 500000.0, "rope_scaling": None,
+                 "rms_norm_eps": 1e-5, "hidden_act": "silu", "tie_word_embeddings": False,
+                 "sliding_window": FOGORAX_WINDOW, "layer_types": ["sliding_attention"] * layers}
+        fog = fogorax_config(vocab=vocab, width=w, layers=layers, heads=H, kv_heads=KV, dim=d, ff=ff,
+                             window=FOGORAX_WINDOW, keep_first=FOGORAX_KEEP, side_dim=side,
+                             max_positions=CONTEXT_CAP, share_every=2)
+        nums = {"llama": model_numbers(llama, layers)}
+        # Fogorax: q, gate and output projections in every layer, keys and values in every other
+        # one, three feed-forward matrices, the two small ones of the per-layer input
+        per_layer = w * d * 3 * H + w * d * KV + 3 * w * ff + 2 * w * side
+        nums["fogorax"] = {"linear_params": layers * per_layer, "head_params": vocab * w,
+                           "kv_values_per_token": layers * KV * d, "attn_hd": H * d, "layers": layers}
+        for model, cfg in (("llama", llama), ("fogorax", fog)):
+            need = batch * (prompt_len + steps + warmup + early_tokens(batch, prompt_len) + 32)
+            engine = build_engine(cfg, dtype, batch, max(need, PREFILL_TOKENS + 64), use_graphs=use_graphs)
+            r = decode_run(engine, vocab, batch, prompt_len, steps, warmup)
+            ctx = min(r["mean_ctx"], FOGORAX_WINDOW + FOGORAX_KEEP)
+            s = prefill_run(engine, vocab, PREFILL_TOKENS, repeats=2)
+            out[f"{name}_{model}"] = {
+                "decode_ms": round(r["ms_per_step"], 4), "decode_tok_s": round(r["tok_s"], 1),
+                "decode_hbm_frac": round(decode_bytes(engine, nums[model], elem, batch, ctx)
+                                         / (r["seconds"] / steps) / 1e9 / HBM_PEAK_GBS, 4),
+                "prefill_tok_s": round(PREFILL_TOKENS / s, 1), "prefill_ms": round(s * 1e3, 3),
+                "prefill_frac": round(prefill_flops(nums[model], PREFILL_TOKENS) / s / MFMA_PEAK[dtype], 4)}
+            del engine
+            torch.cuda.empty_cache()
+    return out
+
+
 def model_numbers(cfg, layers_run):
     h, H, KV, d, I, V = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
                          cfg["head_dim"], cfg["intermediate_size"], cfg["vocab_size"])
@@ -399,14 +454,15 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--decode-run-steps", type=int, default=None,
                     help="decode steps the device takes between two looks of the host (engine default: 8)")
-    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed", "burst", "products"], default="all",
+    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed", "burst", "products", "fogorax"], default="all",
                     help="for profiles: only the decode steps at --batch, or only the prefill; "
                          "mixed: --batch requests with prompts of 128 to 4,096 tokens, chunked "
                          "prefill beside decode steps, --steps new tokens each; burst: the "
                          "workload of the reference's own serving benchmark (48 short requests "
                          "at once, 16 sequences a step), for --preset small or any other; "
                          "products: the four matrix products of a layer alone at --batch rows "
-                         "(launch to launch, so short ones show the host's time)")
+                         "(launch to launch, so short ones show the host's time); fogorax: the "
+                         "Fogorax design at a few layer sizes beside a Llama model of equal sizes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -415,6 +471,17 @@ def main() -> int:
     import torch
     import kvforge_amd
 
+    if args.phase == "fogorax":
+        steps = min(args.steps, 64)
+        print(json.dumps({"phase": "fogorax", "dtype": args.dtype, "batch": args.batch,
+                          "prompt_len": args.prompt_len, "steps": steps, "window": FOGORAX_WINDOW,
+                          "keep_first": FOGORAX_KEEP, "prefill_tokens": PREFILL_TOKENS,
+                          "sizes": {n: {"width": w, "heads": H, "kv_heads": KV, "head_dim": d, "ff": ff,
+                                        "layers": L, "vocab": V, "side_dim": sd}
+                                    for n, w, H, KV, d, ff, L, V, sd in FOGORAX_SIZES},
+                          **fogorax_points(args.dtype, args.batch, args.prompt_len, steps,
+                                           min(args.warmup, 8), not args.no_graphs)}))
+        return 0
     if args.preset == "small" and args.phase != "burst":
         print("--preset small goes with --phase burst")
         return 2

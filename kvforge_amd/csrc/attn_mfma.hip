@@ -74,6 +74,10 @@ struct MArgs {
   float scale;
   unsigned bs_magic;  // floor(2^32 / bs) + 1: key / bs == mulhi(key, bs_magic) while key * bs < 2^32
   const float* slopes;  // null, or one number per q head: slopes[h] * (key - query position) is added to a score
+  // null, or an output gate [tokens, gate_stride >= H * d]: element e of head h of a token's
+  // output is multiplied by sigmoid(gate[token, h * d + e]) as it is stored
+  const bf16_t* gate;
+  int gate_stride;
 };
 
 // A walk over the blocks of 32 keys that a range of rows sees: blocks counted from `first` up to
@@ -281,6 +285,18 @@ __device__ __forceinline__ uint2 pack4(const f32x4& v, float f) {
   pk.x = static_cast<uint32_t>(f32_to_bf16(v[0] * f)) | (static_cast<uint32_t>(f32_to_bf16(v[1] * f)) << 16);
   pk.y = static_cast<uint32_t>(f32_to_bf16(v[2] * f)) | (static_cast<uint32_t>(f32_to_bf16(v[3] * f)) << 16);
   return pk;
+}
+
+// The same through an output gate: g points at the four gate values of the four outputs (or is null).
+__device__ __forceinline__ uint2 pack4_gated(const f32x4& v, float f, const bf16_t* g) {
+  if (!g) return pack4(v, f);
+  const uint2 r = *reinterpret_cast<const uint2*>(g);
+  const float z[4] = {__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u),
+                      __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u)};
+  f32x4 o;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = v[i] * f / (1.f + __expf(-z[i]));
+  return pack4(o, 1.f);
 }
 
 // Sets up the rows of `RT` tiles starting at `first_tile`; returns the positions they span.
@@ -566,8 +582,11 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
     if (!rows.ok[rt]) continue;
     const float inv = l > 0.f ? 1.f / l : 0.f;
     bf16_t* o = out + static_cast<size_t>(q0 + rows.tok[rt]) * a.o_stride + rows.head[rt] * D + 4 * kg;
+    const bf16_t* g = a.gate ? a.gate + static_cast<size_t>(q0 + rows.tok[rt]) * a.gate_stride + rows.head[rt] * D + 4 * kg
+                             : nullptr;
 #pragma unroll
-    for (int t = 0; t < DT; ++t) *reinterpret_cast<uint2*>(o + t * 16) = pack4(acc[rt][t], inv);
+    for (int t = 0; t < DT; ++t)
+      *reinterpret_cast<uint2*>(o + t * 16) = pack4_gated(acc[rt][t], inv, g ? g + t * 16 : nullptr);
   }
   __syncthreads();  // the staging buffers are free for the next item
   }  // part
@@ -751,7 +770,8 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
     const int e0 = t * 16 + 4 * kg;
     if (a.splits == 1)
       *reinterpret_cast<uint2*>(out + static_cast<size_t>(q0 + rows.tok[0]) * a.o_stride + head * D + e0) =
-          pack4(o, inv);
+          pack4_gated(o, inv, a.gate ? a.gate + static_cast<size_t>(q0 + rows.tok[0]) * a.gate_stride + head * D + e0
+                                     : nullptr);
     else
       *reinterpret_cast<f32x4*>(part_acc + slot * D + e0) = o;
   }
@@ -765,7 +785,8 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
 __global__ __launch_bounds__(64) void attn_split_combine_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml,
     const int* __restrict__ seq_ids, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
-    bf16_t* __restrict__ out, int H, int D, int splits, int o_stride, int n_seqs) {
+    bf16_t* __restrict__ out, int H, int D, int splits, int o_stride, int n_seqs,
+    const bf16_t* __restrict__ gate, int gate_stride) {
   const int seq = seq_ids ? seq_ids[blockIdx.x] : static_cast<int>(blockIdx.x);
   if (seq < 0 || seq >= n_seqs) return;
   const int head = blockIdx.y, lane = threadIdx.x;
@@ -792,7 +813,9 @@ __global__ __launch_bounds__(64) void attn_split_combine_kernel(
     for (int s = 0; s < splits; ++s)
       v += part_acc[(slot0 + s) * D + e] *
            __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, c), s));
-    out[static_cast<size_t>(tok) * o_stride + head * D + e].bits = f32_to_bf16(v * inv);
+    float r = v * inv;
+    if (gate) r /= 1.f + __expf(-bf16_to_f32(gate[static_cast<size_t>(tok) * gate_stride + head * D + e].bits));
+    out[static_cast<size_t>(tok) * o_stride + head * D + e].bits = f32_to_bf16(r);
   }
 }
 
@@ -936,9 +959,10 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
                                      const int* work, int num_work, int rows_per_item, void* out, int H, int KV, int d,
                                      int bs, int nb, int table_stride, int q_stride, int o_stride,
                                      int window, int keep, int n_seqs, float scale, const float* slopes,
-                                     hipStream_t s) {
+                                     const void* gate, int gate_stride, hipStream_t s) {
   if (num_work <= 0) return 0;
-  if (keep < 0) return static_cast<int>(hipErrorInvalidValue);
+  if (keep < 0 || (gate && (gate_stride % 4 != 0 || gate_stride < H * d || reinterpret_cast<uintptr_t>(gate) % 8 != 0)))
+    return static_cast<int>(hipErrorInvalidValue);
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0)
     return static_cast<int>(hipErrorInvalidValue);
   const int row_tiles = rows_per_item / (WAVES * 16);
@@ -947,7 +971,8 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
   // workgroups go to consecutive XCDs, so with eight kv heads every XCD walks the keys and values
   // of one head and finds them in its own L2 after the first workgroup has brought them in.
   const int kv_fastest = num_work <= 65535 ? 1 : 0;
-  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, keep, kv_fastest, scale, magic_of(bs), slopes};
+  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, keep, kv_fastest, scale, magic_of(bs), slopes,
+                static_cast<const bf16_t*>(gate), gate_stride};
   const dim3 grid = kv_fastest ? dim3(KV, num_work) : dim3(num_work, KV);
   switch (d / 16) {
 #define GO(DT) \
@@ -967,13 +992,15 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
                                     int num_seqs, int H, int KV, int d, int bs, int nb,
                                     int table_stride, int q_stride, int o_stride, int window,
                                     int keep, int n_seqs, int splits, float scale, const float* slopes,
-                                    hipStream_t s) {
+                                    const void* gate, int gate_stride, hipStream_t s) {
   if (num_seqs <= 0) return 0;
-  if (keep < 0) return static_cast<int>(hipErrorInvalidValue);
+  if (keep < 0 || (gate && (gate_stride % 4 != 0 || gate_stride < H * d || reinterpret_cast<uintptr_t>(gate) % 8 != 0)))
+    return static_cast<int>(hipErrorInvalidValue);
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0 || splits < 1 ||
       splits > KVF_WAVE || (splits > 1 && (!part_acc || !part_ml)))
     return static_cast<int>(hipErrorInvalidValue);
-  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, keep, 0, scale, magic_of(bs), slopes};
+  const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, keep, 0, scale, magic_of(bs), slopes,
+                static_cast<const bf16_t*>(gate), gate_stride};
   const int G = H / KV, chunks = (G + 15) / 16;
   if (num_seqs > 65535) return static_cast<int>(hipErrorInvalidValue);
   const dim3 grid(KV * chunks, num_seqs, splits);
@@ -990,6 +1017,6 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
   if (err || splits == 1) return err;
   hipLaunchKernelGGL(attn_split_combine_kernel, dim3(num_seqs, H), dim3(64), 0, s, part_acc,
                      part_ml, seq_ids, cu_q, ctx_lens, static_cast<bf16_t*>(out), H, d, splits,
-                     o_stride, n_seqs);
+                     o_stride, n_seqs, static_cast<const bf16_t*>(gate), gate_stride);
   return kvf_last_error();
 }

@@ -786,3 +786,90 @@ KVF_EXPORT int kvf_token_side_bf16(TOKEN_SIDE_DECL) {
   return token_side_launch<bf16_t, bf16_t>(x, bias, owed, tokens, side, gate, proj, w, eps, n, h, dim,
                                            vocab, side_stride, col0, s);
 }
+
+// ----------------------------------------------------------------------------- the same, in pieces
+// With many rows the two products of the per-layer token input go to the matrix kernels, and
+// three row-wise kernels stand around them:
+//   settle_cast: x[m] += bias + owed[m] (either may be null); copy[m] = x[m] in T (copy may be null)
+//   side_gate:   g[m, j] = gelu_tanh(a[m, j]) * side[token[m], col0 + j]
+//   rms_add:     x[m] += y[m] * rsqrt(mean(y[m]^2) + eps) * w
+template <typename T, typename D>
+__global__ void settle_cast_kernel(float* __restrict__ x, const float* __restrict__ bias,
+                                   const D* __restrict__ owed, T* __restrict__ copy, int h, size_t total) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  float v = x[i];
+  if (bias) v += bias[i % h];
+  if (owed) v += Elem<D>::load(owed + i);
+  if (bias || owed) x[i] = v;
+  if (copy) Elem<T>::store(copy + i, v);
+}
+template <typename T, typename D>
+static int settle_cast_launch(float* x, const float* bias, const void* owed, void* copy, int m, int h,
+                              hipStream_t s) {
+  const size_t total = static_cast<size_t>(m) * h;
+  if (total == 0 || (!bias && !owed && !copy)) return 0;
+  hipLaunchKernelGGL((settle_cast_kernel<T, D>), dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256),
+                     0, s, x, bias, static_cast<const D*>(owed), static_cast<T*>(copy), h, total);
+  return kvf_last_error();
+}
+KVF_EXPORT int kvf_settle_cast_f32(float* x, const float* bias, const void* owed, int owed_f32, void* copy,
+                                   int m, int h, hipStream_t s) {
+  (void)owed_f32;
+  return settle_cast_launch<float, float>(x, bias, owed, copy, m, h, s);
+}
+KVF_EXPORT int kvf_settle_cast_bf16(float* x, const float* bias, const void* owed, int owed_f32, void* copy,
+                                    int m, int h, hipStream_t s) {
+  if (owed_f32) return settle_cast_launch<bf16_t, float>(x, bias, owed, copy, m, h, s);
+  return settle_cast_launch<bf16_t, bf16_t>(x, bias, owed, copy, m, h, s);
+}
+
+template <typename T>
+__global__ void side_gate_kernel(const T* __restrict__ a, const int* __restrict__ tokens,
+                                 const T* __restrict__ side, T* __restrict__ g, int dim, int vocab,
+                                 int side_stride, int col0, size_t total) {
+  const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t m = idx / dim;
+  const int j = static_cast<int>(idx - m * dim);
+  const int tok = tokens[m];
+  float v = 0.f;
+  if (tok >= 0 && tok < vocab)
+    v = gelu_tanh_f(Elem<T>::load(a + idx)) * Elem<T>::load(side + static_cast<size_t>(tok) * side_stride + col0 + j);
+  Elem<T>::store(g + idx, v);
+}
+template <typename T>
+static int side_gate_launch(const void* a, const int* tokens, const void* side, void* g, int m, int dim,
+                            int vocab, int side_stride, int col0, hipStream_t s) {
+  const size_t total = static_cast<size_t>(m) * dim;
+  if (total == 0) return 0;
+  hipLaunchKernelGGL(side_gate_kernel<T>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, s,
+                     static_cast<const T*>(a), tokens, static_cast<const T*>(side), static_cast<T*>(g), dim,
+                     vocab, side_stride, col0, total);
+  return kvf_last_error();
+}
+KVF_EXPORT int kvf_side_gate_f32(const void* a, const int* t, const void* side, void* g, int m, int dim,
+                                 int vocab, int ss, int col0, hipStream_t s) {
+  return side_gate_launch<float>(a, t, side, g, m, dim, vocab, ss, col0, s);
+}
+KVF_EXPORT int kvf_side_gate_bf16(const void* a, const int* t, const void* side, void* g, int m, int dim,
+                                  int vocab, int ss, int col0, hipStream_t s) {
+  return side_gate_launch<bf16_t>(a, t, side, g, m, dim, vocab, ss, col0, s);
+}
+
+__global__ __launch_bounds__(256) void rms_add_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                      const float* __restrict__ w, float eps, int h) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  float* xr = x + static_cast<size_t>(m) * h;
+  const float* yr = y + static_cast<size_t>(m) * h;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) ss = fmaf(yr[i], yr[i], ss);
+  const float r = rsqrtf(block_sum(ss, scratch) / static_cast<float>(h) + eps);
+  for (int i = threadIdx.x; i < h; i += blockDim.x) xr[i] = fmaf(yr[i] * r, w[i], xr[i]);
+}
+KVF_EXPORT int kvf_rms_add(float* x, const float* y, const float* w, float eps, int m, int h, hipStream_t s) {
+  if (m <= 0) return 0;
+  hipLaunchKernelGGL(rms_add_kernel, dim3(m), dim3(256), 0, s, x, y, w, eps, h);
+  return kvf_last_error();
+}

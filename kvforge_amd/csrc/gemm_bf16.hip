@@ -65,6 +65,11 @@ struct RopeEpi {
   bf16_t* k_pages;
   bf16_t* v_pages;
   int H, KV, d, rot, table_len, block_size, table_stride, num_blocks, write_kv, n_seqs;
+  // EPI 3: the gate's activation (0 silu, 1 the tanh form of gelu) and fp32 biases of the gate and
+  // up columns (by pair, may be null)
+  int act;
+  const float* gate_bias;
+  const float* up_bias;
 };
 
 // Sums that ride along, all bf16 (a workgroup of the fused projection reads every row of A and
@@ -307,7 +312,7 @@ __device__ __forceinline__ void epi_prefetch_b(EpiOperands& op, int n, const Rop
   }
   const int seq = op.page;
   int page = -1;
-  if (head >= rp.H && rp.write_kv && pos_ok) {
+  if (head >= rp.H && head < rp.H + 2 * rp.KV && rp.write_kv && pos_ok) {
     const int blk = p / rp.block_size;
     if (seq >= 0 && seq < rp.n_seqs && blk < rp.table_stride)
       page = rp.block_table[static_cast<size_t>(seq) * rp.table_stride + blk];
@@ -348,8 +353,21 @@ __device__ __forceinline__ void store_tile(const f32x4& s, int m, int n, int N, 
   } else if (EPI == 3) {
     // N is even and n a multiple of 4: two (gate, up) pairs
     bf16_t* o = static_cast<bf16_t*>(Cv) + static_cast<size_t>(m) * ldc + n / 2;
-    o[0].bits = f32_to_bf16(s[0] / (1.f + __expf(-s[0])) * s[1]);
-    if (n + 2 < N) o[1].bits = f32_to_bf16(s[2] / (1.f + __expf(-s[2])) * s[3]);
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {
+      if (n + 2 * pr >= N) break;
+      float g = s[2 * pr], u = s[2 * pr + 1];
+      if (rp.gate_bias) g += rp.gate_bias[n / 2 + pr];
+      if (rp.up_bias) u += rp.up_bias[n / 2 + pr];
+      float a;
+      if (rp.act == 1) {
+        const float t = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+        a = 0.5f * g * (1.f + tanhf(t));
+      } else {
+        a = g / (1.f + __expf(-g));
+      }
+      o[pr].bits = f32_to_bf16(a * u);
+    }
   } else {
     // fused q/k/v projection: d is a multiple of 4, so the four columns lie in one head; pairs
     // that are not rotated (v heads, elements past the rotary width, positions off the table)
@@ -367,6 +385,10 @@ __device__ __forceinline__ void store_tile(const f32x4& s, int m, int n, int N, 
     packed.y = static_cast<uint32_t>(f32_to_bf16(o[2])) | (static_cast<uint32_t>(f32_to_bf16(o[3])) << 16);
     if (head < rp.H) {
       *reinterpret_cast<uint2*>(static_cast<bf16_t*>(Cv) + static_cast<size_t>(m) * ldc + n) = packed;
+    } else if (head >= rp.H + 2 * rp.KV) {
+      // columns behind q, k and v (an output gate, say): stored behind q, as they are
+      *reinterpret_cast<uint2*>(static_cast<bf16_t*>(Cv) + static_cast<size_t>(m) * ldc + n -
+                                2 * rp.KV * rp.d) = packed;
     } else if (op.page >= 0 && op.page < rp.num_blocks) {
       const int off = op.pos % rp.block_size;
       if (head < rp.H + rp.KV) {
@@ -745,8 +767,31 @@ KVF_EXPORT int kvf_gemm_bf16(const void* A, int a_type, const void* W, int w_til
   return static_cast<int>(hipErrorInvalidValue);
 }
 
+// The gated pair epilogue (epi 3) with its activation chosen and biases: out[m, j] =
+// act(c[2j] + gate_bias[j]) * (c[2j+1] + up_bias[j]) as bf16 [M, N/2]; act 0 silu, 1 the tanh form
+// of gelu; the biases are fp32 [N/2] and may be null.
+KVF_EXPORT int kvf_gemm_bf16_gated(const void* A, int a_type, const void* W, int w_tiled, void* C,
+                                   int M, int N, int K, int lda, int ldc, float eps, int act,
+                                   const float* gate_bias, const float* up_bias, hipStream_t s) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || N % 4 != 0 || act < 0 || act > 1)
+    return static_cast<int>(hipErrorInvalidValue);
+  RopeEpi rp{};
+  rp.act = act;
+  rp.gate_bias = gate_bias;
+  rp.up_bias = up_bias;
+  const Riders rd{nullptr, nullptr, nullptr};
+  const bf16_t* w = static_cast<const bf16_t*>(W);
+  if (a_type == 0) return launch_rows<0, 3>(A, w, C, M, N, K, lda, ldc, eps, w_tiled, rd, rp, s);
+  if (a_type == 1) return launch_rows<1, 3>(A, w, C, M, N, K, lda, ldc, eps, w_tiled, rd, rp, s);
+  return static_cast<int>(hipErrorInvalidValue);
+}
+
 // Fused q/k/v projection with rotary and cache write.  W: [(H + 2*KV) * d, K] with q and k rows
 // permuted so that rotary pairs are neighbouring rows.  q_out: [M, ldq >= H * d] bf16.
+// extra_cols (a multiple of 4): further rows of W behind q, k and v, whose columns of the product
+// are stored behind q in q_out as they are (ldq >= H * d + extra_cols); KV may then be 0 for a
+// projection without keys and values.
 // a_add (a_type 1 and at most 16 rows only, may be null): bf16 [M, lda], added to A before the
 // norm.
 KVF_EXPORT int kvf_gemm_bf16_qkv_rope(const void* A, int a_type, const void* W, int w_tiled,
@@ -756,16 +801,17 @@ KVF_EXPORT int kvf_gemm_bf16_qkv_rope(const void* A, int a_type, const void* W, 
                                       const float* sin_t, const int* block_table, void* k_pages,
                                       void* v_pages, int H, int KV, int d, int rot, int table_len,
                                       int block_size, int table_stride, int num_blocks,
-                                      int write_kv, int n_seqs, hipStream_t s) {
+                                      int write_kv, int n_seqs, int extra_cols, hipStream_t s) {
   if (M <= 0) return 0;
   if (K <= 0 || K % 8 != 0 || lda % 8 != 0 || d % 4 != 0 || rot % 2 != 0 || rot > d || ldq % 4 != 0 ||
-      (a_add && (a_type != 1 || M > 16)))
+      (a_add && (a_type != 1 || M > 16)) || extra_cols < 0 || extra_cols % 4 != 0 || KV < 0 ||
+      ldq < H * d + extra_cols)
     return static_cast<int>(hipErrorInvalidValue);
   const Riders rd{static_cast<const bf16_t*>(a_add), nullptr, nullptr};
   const RopeEpi rp{positions, seq_of_token, cos_t, sin_t, block_table,
                    static_cast<bf16_t*>(k_pages), static_cast<bf16_t*>(v_pages), H, KV, d, rot,
-                   table_len, block_size, table_stride, num_blocks, write_kv, n_seqs};
-  const int N = (H + 2 * KV) * d;
+                   table_len, block_size, table_stride, num_blocks, write_kv, n_seqs, 0, nullptr, nullptr};
+  const int N = (H + 2 * KV) * d + extra_cols;
   const bf16_t* w = static_cast<const bf16_t*>(W);
   if (a_type == 0) return launch_rows<0, 4>(A, w, q_out, M, N, K, lda, ldq, eps, w_tiled, rd, rp, s);
   if (a_type == 1) return launch_rows<1, 4>(A, w, q_out, M, N, K, lda, ldq, eps, w_tiled, rd, rp, s);

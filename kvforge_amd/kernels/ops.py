@@ -282,6 +282,54 @@ def token_side(x: torch.Tensor, tokens: torch.Tensor, side: torch.Tensor, col0: 
           side.shape[1], int(col0), _stream()), "token_side")
 
 
+def settle_cast(x: torch.Tensor, bias: torch.Tensor | None = None, owed: torch.Tensor | None = None,
+                copy: torch.Tensor | None = None) -> None:
+    """``x[m] += bias + owed[m]`` for the fp32 stream (either may be ``None``), and, with
+    ``copy`` (``[M, h]`` in fp32 or bf16), a copy of the rows as they then are."""
+    _check(x, "x", F32, (None, None))
+    m, h = x.shape
+    if bias is not None:
+        _check(bias, "bias", F32, (h,))
+    kind = copy.dtype if copy is not None else (owed.dtype if owed is not None and owed.dtype == BF16 else F32)
+    if owed is not None:
+        _check(owed, "owed", None, (m, h))
+        if owed.dtype not in (F32, kind):
+            raise KernelError(f"settle_cast: owed must be float32 or {kind}, got {owed.dtype}")
+    if copy is not None:
+        _check(copy, "copy", None, (m, h))
+    f = _fn("elementwise", f"kvf_settle_cast_{_suffix(kind)}",
+            [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p])
+    _ok(f(x.data_ptr(), bias.data_ptr() if bias is not None else None,
+          owed.data_ptr() if owed is not None else None,
+          1 if owed is not None and owed.dtype == F32 else 0,
+          copy.data_ptr() if copy is not None else None, m, h, _stream()), "settle_cast")
+
+
+def side_gate(a: torch.Tensor, tokens: torch.Tensor, side: torch.Tensor, col0: int, out: torch.Tensor) -> None:
+    """``out[m, j] = gelu_tanh(a[m, j]) * side[tokens[m], col0 + j]`` (zeros for a token outside
+    the table)."""
+    m, dim = a.shape
+    _check(a, "a", None, (m, dim))
+    _check(out, "out", a.dtype, (m, dim))
+    _check(side, "side", a.dtype, (None, None))
+    _check(tokens, "tokens", I32, (None,))
+    if tokens.shape[0] < m or not 0 <= col0 <= side.shape[1] - dim:
+        raise KernelError("side_gate: token ids shorter than the batch, or columns outside the table")
+    f = _fn("elementwise", f"kvf_side_gate_{_suffix(a.dtype)}", [c_void_p] * 4 + [c_int] * 5 + [c_void_p])
+    _ok(f(a.data_ptr(), tokens.data_ptr(), side.data_ptr(), out.data_ptr(), m, dim, side.shape[0],
+          side.shape[1], int(col0), _stream()), "side_gate")
+
+
+def rms_add(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+    """``x[m] += y[m] * rsqrt(mean(y[m]^2) + eps) * weight``, all fp32."""
+    _check(x, "x", F32, (None, None))
+    _check(y, "y", F32, tuple(x.shape))
+    _check(weight, "weight", F32, (x.shape[1],))
+    f = _fn("elementwise", "kvf_rms_add", [c_void_p, c_void_p, c_void_p, c_float, c_int, c_int, c_void_p])
+    _ok(f(x.data_ptr(), y.data_ptr(), weight.data_ptr(), float(eps), x.shape[0], x.shape[1], _stream()),
+        "rms_add")
+
+
 # ------------------------------------------------------------------------------ SwiGLU gate
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor, paired: bool = False) -> None:
     """``out[:, i] = silu(gate_i) * up_i`` where the input row holds gate at ``i`` and up at
@@ -600,6 +648,35 @@ def gemm_generic_vector_alus_only(on: bool) -> bool:
     return bool(f(1 if on else 0))
 
 
+def gemm_gated(a: torch.Tensor, w, out: torch.Tensor, activation: str = "silu",
+               gate_bias: torch.Tensor | None = None, up_bias: torch.Tensor | None = None,
+               rms_eps: float | None = None) -> None:
+    """The MFMA weight-streaming product over (gate, up) row pairs of ``w`` with the gate folded
+    into its store: ``out[:, j] = act(c[2j] + gate_bias[j]) * (c[2j+1] + up_bias[j])``,
+    ``out: [M, N/2]`` bf16.  ``activation``: ``"silu"`` or ``"gelu_tanh"``; biases fp32 ``[N/2]`` or
+    ``None``; ``rms_eps`` as in ``gemm_fused``.  Callers check ``bf16_kernel_takes`` first."""
+    rms = rms_eps is not None
+    m, n, k, lda, ldc = _gemm_operands(a, w, out, lambda n: n // 2)
+    if not bf16_kernel_takes(a, w, rms, True):
+        raise KernelError("gemm_gated: operands do not fit the MFMA kernel")
+    if n % 4 or out.dtype != BF16:
+        raise KernelError("gemm_gated: pairs need N in steps of 4 and a bf16 output")
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"gemm_gated: unknown activation {activation!r}; known: {sorted(ACTIVATIONS)}")
+    for b, name in ((gate_bias, "gate_bias"), (up_bias, "up_bias")):
+        if b is not None:
+            _check(b, name, F32, (n // 2,))
+    if m == 0:
+        return
+    f = _fn("gemm_bf16", "kvf_gemm_bf16_gated",
+            [c_void_p, c_int, c_void_p, c_int, c_void_p] + [c_int] * 5 + [c_float, c_int, c_void_p, c_void_p,
+                                                                        c_void_p])
+    wp, tiled = _w_args(w)
+    _ok(f(a.data_ptr(), 1 if rms else 0, wp, tiled, out.data_ptr(), m, n, k, lda, ldc, float(rms_eps or 0.0),
+          ACTIVATIONS[activation], gate_bias.data_ptr() if gate_bias is not None else None,
+          up_bias.data_ptr() if up_bias is not None else None, _stream()), "gemm_gated")
+
+
 def gemm_fused(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rms_eps: float | None = None,
                silu_pairs: bool = False, accumulate: bool = False) -> None:
     """The MFMA weight-streaming product with work folded in at both ends.
@@ -635,17 +712,23 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
                   seq_of_token: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None,
                   block_table: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                   num_heads: int, num_kv_heads: int, head_dim: int, write_kv: bool = True,
-                  rms_eps: float | None = None, a_owed: torch.Tensor | None = None) -> None:
+                  rms_eps: float | None = None, a_owed: torch.Tensor | None = None,
+                  extra_cols: int = 0) -> None:
     """Fused q/k/v projection: ``a @ w.T`` with rotary applied to q and k (neighbouring columns
     are pairs), rotated q stored to ``q_out [M, H*d]`` and rotated k and v written into the
     pages; without tables (``None``) nothing is rotated.  ``rms_eps`` as in ``gemm_fused``.  ``a_owed`` (with ``rms_eps``; bf16, shape and
     strides, counted in elements, of ``a``): a sum still owed to ``a``; the projection is taken of ``a + a_owed``, and
-    ``a`` itself is left as it is."""
+    ``a`` itself is left as it is.  ``extra_cols``: so many further rows of ``w`` behind q, k and v
+    (an output gate, say), whose columns of the product are stored behind q, ``q_out [M, H*d +
+    extra_cols]``; ``num_kv_heads`` may then be 0 for a projection without keys and values."""
     H, KV, d = num_heads, num_kv_heads, head_dim
+    extra = int(extra_cols)
+    if extra < 0 or extra % 4:
+        raise KernelError(f"gemm_qkv_rope: extra_cols must be a non-negative multiple of 4, got {extra}")
     rms = rms_eps is not None
     m, k = a.shape
     _check(a, "a", None, (m, k), contiguous=False)
-    _check(plain_of(w), "w", BF16, ((H + 2 * KV) * d, k))
+    _check(plain_of(w), "w", BF16, ((H + 2 * KV) * d + extra, k))
     if not bf16_kernel_takes(a, w, rms, True) or a.stride(1) != 1:
         raise KernelError("gemm_qkv_rope: operands do not fit the MFMA kernel")
     if a_owed is not None:
@@ -654,7 +737,7 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
         _check(a_owed, "a_owed", BF16, (m, k), contiguous=False)
         if a_owed.stride() != a.stride():
             raise KernelError("gemm_qkv_rope: a_owed must have the strides of a")
-    _check(q_out, "q_out", BF16, (m, H * d))
+    _check(q_out, "q_out", BF16, (m, H * d + extra))
     _check(positions, "positions", I32, (None,))
     _check(seq_of_token, "seq_of_token", I32, (None,))
     if positions.shape[0] < m or seq_of_token.shape[0] < m:
@@ -663,21 +746,23 @@ def gemm_qkv_rope(a: torch.Tensor, w: torch.Tensor, q_out: torch.Tensor, positio
     if d % 4:
         raise KernelError(f"gemm_qkv_rope: head_dim {d} not supported")
     _check(block_table, "block_table", I32, (None, None))
-    _check(k_pages, "k_pages", BF16, (None, KV, None, d))
+    if KV == 0 and write_kv:
+        raise KernelError("gemm_qkv_rope: a projection without keys and values writes no cache")
+    _check(k_pages, "k_pages", BF16, (None, KV if KV else None, None, d))
     nb, _, bs, _ = k_pages.shape
-    _check(v_pages, "v_pages", BF16, (nb, KV, d, bs))
+    _check(v_pages, "v_pages", BF16, (nb, k_pages.shape[1], d, bs))
     if m == 0:
         return
     f = _fn("gemm_bf16", "kvf_gemm_bf16_qkv_rope",
             [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_float]
-            + [c_void_p] * 8 + [c_int] * 10 + [c_void_p])
+            + [c_void_p] * 8 + [c_int] * 11 + [c_void_p])
     wp, tiled = _w_args(w)
     _ok(f(a.data_ptr(), 1 if rms else 0, wp, tiled, q_out.data_ptr(), m, k,
-          a.stride(0) if m > 1 else k, q_out.stride(0) if m > 1 else H * d, float(rms_eps or 0.0),
+          a.stride(0) if m > 1 else k, q_out.stride(0) if m > 1 else H * d + extra, float(rms_eps or 0.0),
           a_owed.data_ptr() if a_owed is not None else None, positions.data_ptr(), seq_of_token.data_ptr(), cos_p, sin_p,
           block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), H, KV, d, rot,
           table_len, bs, block_table.shape[1], nb, 1 if write_kv else 0, block_table.shape[0],
-          _stream()), "gemm_qkv_rope")
+          extra, _stream()), "gemm_qkv_rope")
 
 
 def pick_workspace(rows: int, n: int, device) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
@@ -796,6 +881,16 @@ def _keep_first(window: int, keep_first: int) -> int:
     return keep if int(window) > 0 else 0
 
 
+def _gate_args(gate, q: torch.Tensor, cols: int):
+    """(pointer, row stride) of an output gate, or (None, 0)."""
+    if gate is None:
+        return None, 0
+    _check(gate, "gate", q.dtype, (None, cols), contiguous=False)
+    if gate.shape[0] < q.shape[0] or gate.stride(1) != 1 or gate.stride(0) % 4 or gate.data_ptr() % 8:
+        raise KernelError("attention: the gate needs a row per token, dense rows that start on 8 bytes")
+    return gate.data_ptr(), gate.stride(0)
+
+
 def attention_on_matrix_cores(dtype: torch.dtype, block_size: int) -> bool:
     """The MFMA attention kernels take bf16 and pages of a multiple of 8 tokens; everything else
     (the true 32-bit path above all) runs the vector-ALU kernel."""
@@ -832,7 +927,7 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  work: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
                  head_dim: int, scale: float, window: int = 0,
                  slopes: torch.Tensor | None = None, rows_per_item: int | None = None,
-                 keep_first: int = 0) -> None:
+                 keep_first: int = 0, gate: torch.Tensor | None = None) -> None:
     """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 3]`` rows
     (sequence row, item, item or -1) where a sequence has ``query_len * H/KV`` rows per kv head,
     an item covers ``rows_per_item`` of them (what ``prefill_rows_per_item`` gave when the rows
@@ -840,23 +935,29 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     one workgroup in turn; rows start in the order given (the longest walks first).  ``v_pages`` are transposed:
     ``[num_blocks, KV, head_dim, block_size]``.  ``slopes``: fp32 ``[H]``; the score of key ``j``
     for a query at position ``p`` of head ``h`` then is ``scale * q.k + slopes[h] * (j - p)``.
-    ``keep_first``: with a window, the first so many keys of a sequence stay visible behind it."""
+    ``keep_first``: with a window, the first so many keys of a sequence stay visible behind it.
+    ``gate`` (``[tokens, H*d]``, dense rows, type of ``q``): an output gate; what is stored is the
+    attention output times ``sigmoid(gate)``, element by element, in the matrix-core kernels'
+    store (the 32-bit kernels take no gate: their caller runs ``sigmoid_gate`` behind them)."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     _check(work, "work", I32, (None, 3))
     keep = _keep_first(window, keep_first)
+    gp, gs = _gate_args(gate, q, H * d)
     sl = _slopes_ptr(slopes, H, q)
     nb, _, bs, _ = k_pages.shape
     if rows_per_item is None:
         rows_per_item = prefill_rows_per_item(q.dtype, d, bs)
     if attention_on_matrix_cores(q.dtype, bs):
         f = _fn("attn_mfma", "kvf_attn_mfma_prefill",
-                [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 11 + [c_float, c_void_p, c_void_p])
+                [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 11 + [c_float, c_void_p, c_void_p, c_int, c_void_p])
         _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
               cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(), work.shape[0], int(rows_per_item), out.data_ptr(),
               H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window), keep,
-              n_seqs, float(scale), sl, _stream()), "attn_mfma_prefill")
+              n_seqs, float(scale), sl, gp, gs, _stream()), "attn_mfma_prefill")
         return
+    if gate is not None:
+        raise KernelError("attn_prefill: the 32-bit kernel takes no gate; gate its rows afterwards")
     if rows_per_item != prefill_rows_per_item(q.dtype, d, bs):
         raise KernelError(f"attn_prefill: the 32-bit kernel takes items of "
                           f"{prefill_rows_per_item(q.dtype, d, bs)} rows, got {rows_per_item}")
@@ -877,18 +978,20 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                 num_kv_heads: int, head_dim: int, scale: float, window: int = 0, splits: int = 1,
                 workspace: tuple[torch.Tensor, torch.Tensor] | None = None,
                 token_is_seq: bool = False, slopes: torch.Tensor | None = None,
-                keep_first: int = 0) -> None:
+                keep_first: int = 0, gate: torch.Tensor | None = None) -> None:
     """Attention of one-token queries: sequence rows ``seq_ids[:num_seqs]`` (or ``0..num_seqs-1``)
     each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys.  The key
     range may be cut into ``splits`` runs; ``workspace`` then holds fp32 partial accumulators
     (``num_seqs * H * splits * d``) and fp32 (max, sum) pairs (``num_seqs * H * splits * 2``).
     ``token_is_seq``: the caller vouches that ``cu_q[i] == i`` for every sequence (a batch of
     single tokens), which spares the matrix-core kernel a dependent load.  ``slopes``: as in
-    ``attn_prefill``; ``keep_first`` likewise."""
+    ``attn_prefill``; ``keep_first`` and ``gate`` likewise (the matrix-core kernels only: the
+    32-bit path is given no gate, its caller gates the rows afterwards)."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     sl = _slopes_ptr(slopes, H, q)
     keep = _keep_first(window, keep_first)
+    gp, gs = _gate_args(gate, q, H * d)
     if token_is_seq and seq_ids is not None:
         raise KernelError("attn_decode: token_is_seq is for batches where every sequence decodes")
     if seq_ids is not None:
@@ -910,6 +1013,8 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
         if pa.numel() < num_seqs * H * splits * d or pm.numel() < num_seqs * H * splits * 2:
             raise KernelError("attn_decode: workspace too small")
     if not attention_on_matrix_cores(q.dtype, bs):
+        if gate is not None:
+            raise KernelError("attn_decode: the 32-bit kernel takes no gate; gate its rows afterwards")
         f = _fn("attn_generic", "kvf_attn_generic_decode",
                 [c_int] + [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p])
         _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
@@ -920,14 +1025,14 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
               int(window), keep, n_seqs, int(splits), float(scale), sl, _stream()), "attn_generic_decode")
         return
     f = _fn("attn_mfma", "kvf_attn_mfma_decode",
-            [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p])
+            [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p, c_int, c_void_p])
     _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
           seq_ids.data_ptr() if seq_ids is not None else None,
           None if token_is_seq else cu_q.data_ptr(),
           ctx_lens.data_ptr(), out.data_ptr(), pa.data_ptr() if pa is not None else None,
           pm.data_ptr() if pm is not None else None, num_seqs, H, KV, d, bs, nb,
           block_table.shape[1], q.stride(0), out.stride(0), int(window), keep, n_seqs, int(splits),
-          float(scale), sl, _stream()), "attn_mfma_decode")
+          float(scale), sl, gp, gs, _stream()), "attn_mfma_decode")
 
 
 # ------------------------------------------------------------------------------ sampling

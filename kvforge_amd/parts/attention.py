@@ -200,13 +200,14 @@ class PagedAttention(Mixer):
         (the kernel that fuses the three has no place for it) and keeps its norm a kernel."""
 
     def _hooked(self) -> bool:
-        """Whether projection, rotation + cache write and attention run as kernels of their
-        own: a variant with a hook between them, a gate, or no keys and values of its own."""
-        return (type(self).after_projection is not PagedAttention.after_projection
-                or self.gated or not self.own_kv)
+        return type(self).after_projection is not PagedAttention.after_projection
+
+    def _plain(self) -> bool:
+        """Whether the product holds q, k and v and nothing else."""
+        return self.own_kv and not self.gated
 
     def absorb_norm(self, norm) -> bool:
-        if self._hooked():
+        if self._hooked() or not self._plain():
             return False
         if self.norm_eps is not None or not getattr(norm, "foldable_into", lambda m: False)(self.w_qkv):
             return False
@@ -311,13 +312,17 @@ class PagedAttention(Mixer):
                 owed = None
         else:
             step.settle()
+        g0 = H * d     # where the gate's columns begin in a row of qkv
         if fused:
-            # one kernel: (norm,) projection, rotary, cache write
-            qkv = ws.buf("q_rot", (n, H * d), act)
+            # one kernel: (norm,) projection, rotary, cache write; a gate's columns land behind q
+            extra = H * d if self.gated else 0
+            qkv = ws.buf("q_rot", (n, H * d + extra), act)
             ops.gemm_qkv_rope(x, self.w_qkv, qkv, step.positions, step.seq_of_token, cos, sin, table,
-                              layer.k_pages, layer.v_pages, H, KV, d, write_kv=layer.owns_cache,
-                              rms_eps=rms, a_owed=owed)
+                              layer.k_pages, layer.v_pages, H, KV if self.own_kv else 0, d,
+                              write_kv=layer.owns_cache and self.own_kv, rms_eps=rms, a_owed=owed,
+                              extra_cols=extra)
         else:
+            g0 = (H + (2 * KV if self.own_kv else 0)) * d
             qkv = ws.buf("qkv", (n, self.w_qkv.shape[0]), act)
             ops.gemm(x, self.w_qkv, qkv)
             self.after_projection(qkv, step)
@@ -329,10 +334,13 @@ class PagedAttention(Mixer):
         window = self.window or 0
         bs = layer.k_pages.shape[2]
         work, rows_per_item = self._prefill_work(step, act, bs)
+        gate = qkv[:, g0:g0 + H * d] if self.gated else None
+        # the matrix-core kernels gate their output as they store it
+        gate_in_kernel = gate if gate is not None and ops.attention_on_matrix_cores(act, bs) else None
         if work is not None:
             ops.attn_prefill(qkv, layer.k_pages, layer.v_pages, table, step.cu_q, step.ctx_lens,
                              work, out, H, KV, d, self.scale, window, self.slopes, rows_per_item,
-                             keep_first=self.keep_first)
+                             keep_first=self.keep_first, gate=gate_in_kernel)
         if step.n_decode:
             splits = self._decode_cuts(step, ops.attention_on_matrix_cores(act, bs))
             workspace = None
@@ -343,8 +351,7 @@ class PagedAttention(Mixer):
                             step.n_decode, step.cu_q, step.ctx_lens, out, H, KV, d, self.scale,
                             window, splits, workspace,
                             token_is_seq=step.decode_seq_ids is None and work is None,
-                            slopes=self.slopes, keep_first=self.keep_first)
-        if self.gated:
-            g0 = (H + (2 * KV if self.own_kv else 0)) * d
-            ops.sigmoid_gate(out, qkv[:, g0:g0 + H * d])
+                            slopes=self.slopes, keep_first=self.keep_first, gate=gate_in_kernel)
+        if gate is not None and gate_in_kernel is None:
+            ops.sigmoid_gate(out, gate)
         add_product(step, out, self.w_o, residual, owed=owed)

@@ -148,11 +148,15 @@ class GatedFeedForward(SwiGLU):
         n = x.shape[0]
         ws, dt = step.ws, step.act_dtype
         step.settle()
-        gu = ws.buf("gate_up", (n, 2 * self.inter), dt)
-        ops.gemm(x, self.w_gate_up, gu)
         act = ws.buf("ffn_act", (n, self.inter), dt)
-        ops.gated_act(gu, act, self.activation, paired=True, gate_bias=self.gate_bias,
-                      up_bias=self.up_bias)
+        if ops.bf16_kernel_takes(x, self.w_gate_up, False, True) and self.inter % 2 == 0:
+            # one kernel: gate/up projection, biases, activation, gate
+            ops.gemm_gated(x, self.w_gate_up, act, self.activation, self.gate_bias, self.up_bias)
+        else:
+            gu = ws.buf("gate_up", (n, 2 * self.inter), dt)
+            ops.gemm(x, self.w_gate_up, gu)
+            ops.gated_act(gu, act, self.activation, paired=True, gate_bias=self.gate_bias,
+                          up_bias=self.up_bias)
         add_product(step, act, self.w_down, residual)
         if self.down_bias is not None and not self.defer_down_bias:
             step.settle()

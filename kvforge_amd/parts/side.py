@@ -12,7 +12,9 @@ from kvforge_amd.parts.base import Part, WeightSpec
 class TokenSideInput(Part):
     """With ``e = table[token, first_col : first_col + dim]`` and the fp32 stream row ``x``:
     ``y = proj @ (gelu_tanh(gate @ x) * e)`` and ``x += y * rsqrt(mean(y^2) + eps) * weight`` (an RMS
-    norm with a weight per coordinate), all in one kernel with fp32 sums.
+    norm with a weight per coordinate).  Few rows take one kernel with fp32 sums throughout; many
+    rows send the two products to the matrix kernels (in the engine's type, fp32 sums) with
+    three row-wise kernels around them.
 
     ``table_name``: checkpoint name of the table ``[vocab, table_cols]`` that the layers share;
     ``gate [dim, hidden]``, ``proj [hidden, dim]`` and ``norm [hidden]`` live under the prefix.
@@ -44,7 +46,7 @@ class TokenSideInput(Part):
         self.weight = tensors[self._name("norm")].float().contiguous()
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
-        return {"elementwise"}
+        return {"elementwise", "gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())
 
     def num_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in (self.gate, self.proj, self.weight) if t is not None)
@@ -52,7 +54,27 @@ class TokenSideInput(Part):
     def held_tensors(self) -> list[torch.Tensor]:
         return [t for t in (self.table, self.gate, self.proj, self.weight) if t is not None]
 
+    # rows up to which one kernel does everything, a workgroup per row with the two small
+    # matrices read through the caches; beyond, the two products go to the matrix kernels
+    FUSED_MAX_ROWS = 32
+
     def forward(self, residual: torch.Tensor, step, bias: torch.Tensor | None = None) -> None:
         """``bias`` (fp32 ``[hidden]``): a bias the stream is still owed, besides ``step.owed``."""
-        ops.token_side(residual, step.token_ids, self.table, self.first_col, self.gate, self.proj,
-                       self.weight, self.eps, bias=bias, owed=step.take_owed(residual))
+        n = residual.shape[0]
+        owed = step.take_owed(residual)
+        if n <= self.FUSED_MAX_ROWS:
+            ops.token_side(residual, step.token_ids, self.table, self.first_col, self.gate, self.proj,
+                           self.weight, self.eps, bias=bias, owed=owed)
+            return
+        ws, dt = step.ws, self.gate.dtype
+        x = residual
+        if dt != torch.float32:
+            x = ws.buf("side_rows", (n, self.hidden), dt)
+        ops.settle_cast(residual, bias, owed, x if x is not residual else None)
+        a = ws.buf("side_a", (n, self.dim), dt)
+        ops.gemm(x, self.gate, a)
+        g = ws.buf("side_g", (n, self.dim), dt)
+        ops.side_gate(a, step.token_ids, self.table, self.first_col, g)
+        y = ws.buf("side_y", (n, self.hidden), torch.float32)
+        ops.gemm(g, self.proj, y)
+        ops.rms_add(residual, y, self.weight, self.eps)

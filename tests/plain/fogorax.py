@@ -26,8 +26,9 @@ def stored(x: torch.Tensor, store: torch.dtype | None) -> torch.Tensor:
     """``x`` as it is after a trip through memory in type ``store`` (rounded and widened
     again), or unchanged for ``None``.  ``forward(..., store=torch.bfloat16)`` rounds so every
     tensor that an engine serving in bfloat16 may keep in 16 bits between two operations
-    (normalised rows, projections, attention outputs, activations), and nothing else: the
-    stream, norms, scores and softmax stay as they are.  What that run differs from the
+    (normalised rows, projections and other products, attention outputs, activations, the
+    stream's rows where a product reads them), and nothing else: the stream itself, norms, scores
+    and softmax stay as they are.  What that run differs from the
     unrounded one by is the size of rounding alone."""
     return x if store is None else x.to(store).to(x.dtype)
 
@@ -94,14 +95,15 @@ def dense_ff(h: torch.Tensor, w: dict, p: str, store: torch.dtype | None = None)
     """``down(gelu(gate h + b) * (up h + b)) + b`` with tensors ``p.gate``, ``p.gate.b`` ..."""
     a = gelu_tanh(stored(h @ w[p + ".gate"].T, store) + w[p + ".gate.b"])
     b = stored(h @ w[p + ".up"].T, store) + w[p + ".up.b"]
-    return stored(a * b, store) @ w[p + ".down"].T + w[p + ".down.b"]
+    return stored(stored(a * b, store) @ w[p + ".down"].T, store) + w[p + ".down.b"]
 
 
 def token_side(x: torch.Tensor, side_rows: torch.Tensor, gate: torch.Tensor, proj: torch.Tensor,
-               weight: torch.Tensor, eps: float) -> torch.Tensor:
+               weight: torch.Tensor, eps: float, store: torch.dtype | None = None) -> torch.Tensor:
     """What the per-layer token input adds to the stream ``x``: ``side_rows [T, dim]`` are the
     layer's part of each token's row of the side table."""
-    y = (gelu_tanh(x @ gate.T) * side_rows) @ proj.T
+    a = stored(stored(x, store) @ gate.T, store)
+    y = stored(gelu_tanh(a) * side_rows, store) @ proj.T
     return rms(y, eps) * weight
 
 
@@ -138,7 +140,7 @@ def forward(config: dict, weights: dict, tokens, dtype: torch.dtype = torch.floa
             heads = stored(gated_attention(q, k, v, torch.full_like(g, float("inf")), H, G, d, dv,
                                            float(m["scale"]), mask), store)
             heads = stored(heads * torch.sigmoid(g), store)
-        delta = heads @ w[p + ".mix.o"].T
+        delta = stored(heads @ w[p + ".mix.o"].T, store)
         if layer.get("mlp") is not None:
             if layer["mlp"]["kind"] != "dense":
                 raise ValueError(f"layer {i}: unknown feed-forward {layer['mlp']['kind']!r}")
@@ -146,7 +148,7 @@ def forward(config: dict, weights: dict, tokens, dtype: torch.dtype = torch.floa
         x = x + delta
         if sdim:
             x = x + token_side(x, w["side.embed"][tok][:, i * sdim:(i + 1) * sdim],
-                               w[p + ".side.gate"], w[p + ".side.proj"], w[p + ".side.norm"], eps)
+                               w[p + ".side.gate"], w[p + ".side.proj"], w[p + ".side.norm"], eps, store)
         if layers_out is not None:
             layers_out.append(x.clone())
     return stored(scalar_norm(x, w["final.norm"], eps), store) @ w["head"].T

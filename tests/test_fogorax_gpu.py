@@ -153,6 +153,122 @@ def test_token_side(dtype, h, dim, extras):
     torch.testing.assert_close(got.cpu(), want, atol=1e-4, rtol=1e-4)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("extras", ["both", "none", "bias", "owed"])
+def test_token_side_in_pieces_for_many_rows(dtype, extras):
+    """The part's two routes give the same stream: one kernel for few rows, the matrix kernels
+    with three row-wise kernels around them for many."""
+    from kvforge_amd.engine.batch import Step, Workspace
+    from kvforge_amd.parts import TokenSideInput
+
+    n, h, dim, vocab = 70, 96, 24, 50
+    part = TokenSideInput("l1.side", h, dim, vocab, "side.embed", 3 * dim, dim, 1e-5)
+    part.load({"side.embed": rand(vocab, 3 * dim, seed=2).to(dtype).to(DEV),
+               "l1.side.gate": rand(dim, h, seed=3, scale=h ** -0.5).to(dtype).to(DEV),
+               "l1.side.proj": rand(h, dim, seed=4).to(dtype).to(DEV),
+               "l1.side.norm": (1.0 + rand(h, seed=5, scale=0.1)).to(dtype).to(DEV)})
+    x = rand(n, h, seed=1)
+    bias = rand(h, seed=6).to(DEV) if extras in ("both", "bias") else None
+    owed = rand(n, h, seed=7).to(dtype).to(DEV) if extras in ("both", "owed") else None
+    tokens = torch.randint(-1, vocab + 1, (n,), generator=torch.Generator().manual_seed(8)).int()
+    got = []
+    for limit in (1 << 30, 0):
+        part.FUSED_MAX_ROWS = limit
+        step = Step()
+        step.ws, step.act_dtype, step.device, step.token_ids = Workspace(DEV), dtype, DEV, tokens.to(DEV)
+        res = x.clone().to(DEV)
+        if owed is not None:
+            step.owe(res, owed)
+        part.forward(res, step, bias=bias)
+        assert step.owed is None
+        got.append(res.cpu())
+    base = x + (bias.cpu() if bias is not None else 0.0) + (owed.float().cpu() if owed is not None else 0.0)
+    known = (tokens >= 0) & (tokens < vocab)
+    rows = part.table.float().cpu()[tokens.clamp(0, vocab - 1).long()][:, dim:2 * dim]
+    want = base + plain.token_side(base, rows, part.gate.float().cpu(), part.proj.float().cpu(),
+                                   part.weight.cpu(), 1e-5) * known[:, None]
+    torch.testing.assert_close(got[0], want, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(got[1], want, **(dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32
+                                                 else dict(atol=4e-2, rtol=4e-2)))
+
+
+@pytest.mark.parametrize("m", [1, 8, 33])
+@pytest.mark.parametrize("activation,bias", [("gelu_tanh", True), ("silu", True), ("gelu_tanh", False)])
+def test_gate_folded_into_the_projection(m, activation, bias):
+    """The weight-streaming product with biases, activation and gate in its store against the
+    product followed by the activation kernel."""
+    k, inter = 96, 70
+    a = rand(m, k, seed=1).bfloat16().to(DEV)
+    w = ops().streamed(rand(2 * inter, k, seed=2, scale=k ** -0.5).bfloat16().to(DEV))
+    bg, bu = (rand(inter, seed=3).to(DEV), rand(inter, seed=4).to(DEV)) if bias else (None, None)
+    got = torch.empty(m, inter, dtype=torch.bfloat16, device=DEV)
+    ops().gemm_gated(a, w, got, activation, bg, bu)
+    c = a.float().cpu() @ w.plain.float().cpu().T
+    g, u = c[:, 0::2] + (bg.cpu() if bias else 0.0), c[:, 1::2] + (bu.cpu() if bias else 0.0)
+    want = (plain.gelu_tanh(g) if activation == "gelu_tanh" else g * torch.sigmoid(g)) * u
+    torch.testing.assert_close(got.float().cpu(), want, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("m", [1, 5, 40])
+@pytest.mark.parametrize("own_kv", [True, False])
+def test_projection_with_cache_write_carries_a_gates_columns(m, own_kv):
+    """Rows of W behind q, k and v come out behind q; without k and v rows nothing is written."""
+    H, KV, d, k, bs = 3, 1, 32, 64, 8
+    kv = KV if own_kv else 0
+    n = (H + 2 * kv) * d + H * d
+    a = rand(m, k, seed=1).bfloat16().to(DEV)
+    w = rand(n, k, seed=2, scale=k ** -0.5).bfloat16().to(DEV)
+    pos = torch.arange(3, 3 + m, dtype=torch.int32, device=DEV)
+    seq_of = torch.zeros(m, dtype=torch.int32, device=DEV)
+    table = torch.arange(8, dtype=torch.int32, device=DEV).flip(0).reshape(1, 8).contiguous()
+    kp = torch.zeros(8, KV, bs, d, dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros(8, KV, d, bs, dtype=torch.bfloat16, device=DEV)
+    out = torch.empty(m, 2 * H * d, dtype=torch.bfloat16, device=DEV)
+    ops().gemm_qkv_rope(a, ops().streamed(w), out, pos, seq_of, None, None, table, kp, vp, H, kv, d,
+                        write_kv=own_kv, extra_cols=H * d)
+    c = (a.float() @ w.float().T).cpu()
+    torch.testing.assert_close(out[:, :H * d].float().cpu(), c[:, :H * d], atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(out[:, H * d:].float().cpu(), c[:, n - H * d:], atol=2e-2, rtol=2e-2)
+    if not own_kv:
+        assert float(kp.abs().max()) == 0.0 and float(vp.abs().max()) == 0.0
+        return
+    for t in range(m):
+        p = 3 + t
+        page, off = 7 - p // bs, p % bs
+        torch.testing.assert_close(kp[page, 0, off].float().cpu(), c[t, H * d:(H + 1) * d], atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(vp[page, 0, :, off].float().cpu(), c[t, (H + 1) * d:(H + 2) * d], atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("H,KV,d,bs", [(4, 2, 16, 8), (6, 2, 64, 16), (5, 1, 128, 16)])
+@pytest.mark.parametrize("splits", [1, 3])
+def test_attention_gates_its_output_as_it_stores_it(H, KV, d, bs, splits):
+    """Query runs and single tokens on the matrix cores, the gate read from columns of the
+    buffer that holds q."""
+    dtype, window, keep = torch.bfloat16, 21, 2
+    scale = 1 / math.sqrt(d)
+    for seq_lens, q_lens in (([90, 33, 70], [40, 33, 2]), ([7, 90, 1, 300], [1, 1, 1, 1])):
+        paged = Paged(seq_lens, KV, d, bs, dtype, seed=d)
+        n = sum(q_lens)
+        buf = rand(n, 2 * H * d, seed=d + 1).to(dtype)
+        q = buf[:, :H * d].reshape(n, H, d)
+        cu = torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32)
+        ctx = torch.tensor(seq_lens, dtype=torch.int32)
+        want = masked_reference(paged, q, seq_lens, q_lens, scale, window, keep).reshape(n, H * d)
+        want = want * torch.sigmoid(buf[:, H * d:].float())
+        dev = buf.to(DEV)
+        out = torch.zeros(n, H * d, dtype=dtype, device=DEV)
+        if max(q_lens) > 1:
+            ops().attn_prefill(dev, paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV), cu.to(DEV), ctx.to(DEV),
+                               prefill_work(q_lens, H // KV, dtype, d, bs).to(DEV), out, H, KV, d, scale, window,
+                               keep_first=keep, gate=dev[:, H * d:])
+        else:
+            ws = (torch.empty(n * H * splits * d, device=DEV), torch.empty(n * H * splits * 2, device=DEV))
+            ops().attn_decode(dev, paged.k.to(DEV), paged.v.to(DEV), paged.table.to(DEV), None, n, cu.to(DEV),
+                              ctx.to(DEV), out, H, KV, d, scale, window, splits, ws, keep_first=keep,
+                              gate=dev[:, H * d:])
+        torch.testing.assert_close(out.float().cpu(), want, **tol(dtype))
+
+
 def masked_reference(paged, q, seq_lens, q_lens, scale, window, keep):
     outs, off = [], 0
     for s, (n, ql) in enumerate(zip(seq_lens, q_lens)):
@@ -373,11 +489,14 @@ def close_to_plain(got: torch.Tensor, want: torch.Tensor, dtype, what="", rounde
     ``rounded`` is the plain model run with the roundings a bfloat16 engine may make
     (``plain.forward(store=bfloat16)``), and a row may be off by three times what that run is
     off in the same row (or the fixed share, if that is more).  A lost key, state or page moves a row
-    by about the whole spread."""
+    by about the whole spread, twenty times any of these."""
     err = row_error(got, want)
     limit = torch.full_like(err, 2e-4 if dtype == torch.float32 else 3e-2)
     if rounded is not None and dtype != torch.float32:
-        limit = torch.maximum(limit, 3.0 * row_error(rounded, want))
+        off = row_error(rounded, want)
+        # (the largest of hundreds of rows is a wide-tailed thing: a row is also allowed one and
+        # a half times what the worst row of the rounded run is off)
+        limit = torch.maximum(limit, torch.maximum(3.0 * off, 1.5 * off.max()))
     worst = int((err / limit).argmax())
     assert float(err[worst]) <= float(limit[worst]), (
         f"{what}: position {worst} is off by {float(err[worst]):.3e} of the logits' spread "
