@@ -512,8 +512,10 @@ KVF_EXPORT int kvf_add_positions_bf16(float* x, const void* t, const int* p, int
 // token in the sequence's state slot, after it has read the slot: no other workgroup touches
 // that slot, so reading and writing it need no order between workgroups.  A sequence without a
 // slot (negative: the padding of a captured batch) has no state.
+constexpr int SHIFT_THREADS = 512, SHIFT_KEEP = 8;  // rows up to 4,096 elements live in registers
+
 template <typename T>
-__global__ __launch_bounds__(256) void norm_shift_kernel(
+__global__ __launch_bounds__(SHIFT_THREADS) void norm_shift_kernel(
     const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ mu,
     float* __restrict__ state, const int* __restrict__ slot_ids, const int* __restrict__ seq_of_token,
     const int* __restrict__ cu_q, const int* __restrict__ positions, T* __restrict__ plain,
@@ -531,41 +533,65 @@ __global__ __launch_bounds__(256) void norm_shift_kernel(
   if (slot >= n_slots) slot = -1;
   const float* xr = x + static_cast<size_t>(t) * h;
   const float inv_h = 1.f / static_cast<float>(h);
-
-  float ss = 0.f;
-  for (int i = threadIdx.x; i < h; i += blockDim.x) ss = fmaf(xr[i], xr[i], ss);
-  const float r = rsqrtf(block_sum(ss, scratch) * inv_h + eps);
-
   // where the predecessor comes from: 0 nothing, 1 the row before, 2 the state slot
   const int from = pos <= 0 ? 0 : (!first ? 1 : (slot >= 0 ? 2 : 0));
-  float rp = 0.f;
   const float* xp = xr - h;
-  if (from == 1) {
-    float sp = 0.f;
-    for (int i = threadIdx.x; i < h; i += blockDim.x) sp = fmaf(xp[i], xp[i], sp);
-    rp = rsqrtf(block_sum(sp, scratch) * inv_h + eps);
-  }
   const float* st = slot >= 0 ? state + static_cast<size_t>(slot) * h : nullptr;
+  const bool save = first && slot >= 0;
+  const float* xl = x + static_cast<size_t>(q_last) * h;   // the row whose y goes to the slot
+
+  // Everything a thread needs of its first SHIFT_KEEP elements is asked for before the first
+  // reduction, so that the loads' latencies overlap; elements past them are read where used.
+  float xv[SHIFT_KEEP], pv[SHIFT_KEEP], lv[SHIFT_KEEP], wv[SHIFT_KEEP], mv[SHIFT_KEEP];
+  float ss = 0.f, sp = 0.f, sl = 0.f;
+#pragma unroll
+  for (int k = 0; k < SHIFT_KEEP; ++k) {
+    const int i = threadIdx.x + k * SHIFT_THREADS;
+    const bool in = i < h;
+    xv[k] = in ? xr[i] : 0.f;
+    pv[k] = !in ? 0.f : (from == 1 ? xp[i] : (from == 2 ? st[i] : 0.f));
+    lv[k] = in && save && q_last != t ? xl[i] : 0.f;
+    wv[k] = in ? w[i] : 0.f;
+    mv[k] = in ? mu[i] : 0.f;
+  }
+#pragma unroll
+  for (int k = 0; k < SHIFT_KEEP; ++k) {
+    ss = fmaf(xv[k], xv[k], ss);
+    if (from == 1) sp = fmaf(pv[k], pv[k], sp);
+    sl = fmaf(lv[k], lv[k], sl);
+  }
+  for (int i = threadIdx.x + SHIFT_KEEP * SHIFT_THREADS; i < h; i += SHIFT_THREADS) {
+    ss = fmaf(xr[i], xr[i], ss);
+    if (from == 1) sp = fmaf(xp[i], xp[i], sp);
+    if (save && q_last != t) sl = fmaf(xl[i], xl[i], sl);
+  }
+  // the same order of sums for a row whichever workgroup norms it: a thread's elements in
+  // turn, then the block's tree
+  const float r = rsqrtf(block_sum(ss, scratch) * inv_h + eps);
+  const float rp = from == 1 ? rsqrtf(block_sum(sp, scratch) * inv_h + eps) : 1.f;
+  const float rl = save && q_last != t ? rsqrtf(block_sum(sl, scratch) * inv_h + eps) : r;
+
   T* po = plain + static_cast<size_t>(t) * h;
   T* so = shifted + static_cast<size_t>(t) * h;
-  for (int i = threadIdx.x; i < h; i += blockDim.x) {
+  float* sw = save ? state + static_cast<size_t>(slot) * h : nullptr;
+#pragma unroll
+  for (int k = 0; k < SHIFT_KEEP; ++k) {
+    const int i = threadIdx.x + k * SHIFT_THREADS;
+    if (i >= h) break;
+    const float y = xv[k] * r * wv[k];
+    const float prev = from == 1 ? pv[k] * rp * wv[k] : pv[k];
+    Elem<T>::store(po + i, y);
+    Elem<T>::store(so + i, fmaf(prev - y, mv[k], y));
+    // this thread has read the slot's element that it writes
+    if (save) sw[i] = q_last == t ? y : lv[k] * rl * wv[k];
+  }
+  for (int i = threadIdx.x + SHIFT_KEEP * SHIFT_THREADS; i < h; i += SHIFT_THREADS) {
     const float y = xr[i] * r * w[i];
     const float prev = from == 1 ? xp[i] * rp * w[i] : (from == 2 ? st[i] : 0.f);
     Elem<T>::store(po + i, y);
     Elem<T>::store(so + i, fmaf(prev - y, mu[i], y));
+    if (save) sw[i] = q_last == t ? y : xl[i] * rl * w[i];
   }
-  if (!first || slot < 0) return;
-  // every thread has read the elements of the slot that it is about to write
-  float* sw = state + static_cast<size_t>(slot) * h;
-  if (q_last == t) {
-    for (int i = threadIdx.x; i < h; i += blockDim.x) sw[i] = xr[i] * r * w[i];
-    return;
-  }
-  const float* xl = x + static_cast<size_t>(q_last) * h;
-  float sl = 0.f;
-  for (int i = threadIdx.x; i < h; i += blockDim.x) sl = fmaf(xl[i], xl[i], sl);
-  const float rl = rsqrtf(block_sum(sl, scratch) * inv_h + eps);
-  for (int i = threadIdx.x; i < h; i += blockDim.x) sw[i] = xl[i] * rl * w[i];
 }
 template <typename T>
 static int norm_shift_launch(const float* x, const float* w, const float* mu, float* state,
@@ -574,7 +600,7 @@ static int norm_shift_launch(const float* x, const float* w, const float* mu, fl
                              int n_seqs, int n_slots, hipStream_t s) {
   if (n <= 0) return 0;
   // one block size for every call: the order of a row's sum of squares must not depend on the batch
-  hipLaunchKernelGGL(norm_shift_kernel<T>, dim3(n), dim3(256), 0, s, x, w, mu, state, slot_ids,
+  hipLaunchKernelGGL(norm_shift_kernel<T>, dim3(n), dim3(SHIFT_THREADS), 0, s, x, w, mu, state, slot_ids,
                      seq_of_token, cu_q, positions, static_cast<T*>(plain), static_cast<T*>(shifted), eps,
                      h, n_seqs, n_slots, n);
   return kvf_last_error();
@@ -756,12 +782,124 @@ __global__ __launch_bounds__(256) void token_side_kernel(
     xr[i] = fmaf(acc * r, w[i], row[i]);
   }
 }
+// The same for rows of a multiple of 8 elements (h and dim), 1,024 threads and 16-byte loads: what
+// a decode step runs.  `proj_t` is the projection transposed, [dim, h], so that the lanes of a
+// wave read neighbouring elements of y's row.  The sixteen waves take the rows of `gate` in
+// turn; for y a thread owns eight neighbouring elements and one of JG shares of the sum over
+// dim, the shares are added in LDS in a fixed order.
+template <typename T, typename D>
+__global__ __launch_bounds__(1024) void token_side_wide_kernel(
+    float* __restrict__ x, const float* __restrict__ bias, const D* __restrict__ owed,
+    const int* __restrict__ tokens, const T* __restrict__ side, const T* __restrict__ gate,
+    const T* __restrict__ proj_t, const float* __restrict__ w, float eps, int h, int dim, int vocab,
+    int side_stride, int col0, int CC, int JG) {
+  extern __shared__ __align__(16) float side_lds[];  // [h] the row, [JG][h] shares of y, [dim] g
+  __shared__ float scratch[16];
+  float* row = side_lds;
+  float* part = side_lds + h;
+  float* g = part + static_cast<size_t>(JG) * h;
+  const int m = blockIdx.x, tid = threadIdx.x;
+  const int lane = tid % KVF_WAVE, wave = tid / KVF_WAVE, waves = blockDim.x / KVF_WAVE;
+  float* xr = x + static_cast<size_t>(m) * h;
+  const D* orow = owed ? owed + static_cast<size_t>(m) * h : nullptr;
+  for (int i = tid; i < h; i += blockDim.x) {
+    float v = xr[i];
+    if (bias) v += bias[i];
+    if (orow) v += Elem<D>::load(orow + i);
+    row[i] = v;
+  }
+  __syncthreads();
+  const int tok = tokens[m];
+  const bool known = tok >= 0 && tok < vocab;
+  const T* e = side + static_cast<size_t>(known ? tok : 0) * side_stride + col0;
+  const int chunks = h / 8;
+  // a wave takes four rows of `gate` at a time, so that their loads are in flight together
+  // (rows past dim are read again from row 0 and dropped)
+  constexpr int RB = 4;
+  for (int j0 = wave; j0 < dim; j0 += RB * waves) {
+    float a[RB] = {0.f, 0.f, 0.f, 0.f};
+    for (int c = lane; c < chunks; c += KVF_WAVE) {
+      float v[RB][8];
+#pragma unroll
+      for (int u = 0; u < RB; ++u) {
+        const int j = j0 + u * waves;
+        load8(gate + static_cast<size_t>(j < dim ? j : 0) * h + 8 * c, v[u]);
+      }
+      const float4 r0 = *reinterpret_cast<const float4*>(row + 8 * c);
+      const float4 r1 = *reinterpret_cast<const float4*>(row + 8 * c + 4);
+#pragma unroll
+      for (int u = 0; u < RB; ++u) {
+        float t = a[u];
+        t = fmaf(v[u][0], r0.x, t); t = fmaf(v[u][1], r0.y, t); t = fmaf(v[u][2], r0.z, t); t = fmaf(v[u][3], r0.w, t);
+        t = fmaf(v[u][4], r1.x, t); t = fmaf(v[u][5], r1.y, t); t = fmaf(v[u][6], r1.z, t); t = fmaf(v[u][7], r1.w, t);
+        a[u] = t;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < RB; ++u) {
+      const int j = j0 + u * waves;
+      const float t = wave_sum(a[u]);
+      if (lane == 0 && j < dim) g[j] = known ? gelu_tanh_f(t) * Elem<T>::load(e + j) : 0.f;
+    }
+  }
+  __syncthreads();
+  // shares of y: thread (c, jg) sums g[j] * proj_t[j][8c .. 8c+7] over j = jg, jg + JG, ...
+  const int jg = tid / CC, c0 = tid - jg * CC;
+  if (jg < JG) {
+    for (int c = c0; c < chunks; c += CC) {
+      float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      // four rows of the transposed projection in flight (rows past dim count with g = 0)
+      for (int j0 = jg; j0 < dim; j0 += RB * JG) {
+        float v[RB][8], gj[RB];
+#pragma unroll
+        for (int u = 0; u < RB; ++u) {
+          const int j = j0 + u * JG;
+          load8(proj_t + static_cast<size_t>(j < dim ? j : 0) * h + 8 * c, v[u]);
+          gj[u] = j < dim ? g[j] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < RB; ++u)
+#pragma unroll
+          for (int k = 0; k < 8; ++k) acc[k] = fmaf(v[u][k], gj[u], acc[k]);
+      }
+      float* p = part + static_cast<size_t>(jg) * h + 8 * c;
+      *reinterpret_cast<float4*>(p) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      *reinterpret_cast<float4*>(p + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    }
+  }
+  __syncthreads();
+  float ss = 0.f;
+  for (int i = tid; i < h; i += blockDim.x) {
+    float y = part[i];
+    for (int q = 1; q < JG; ++q) y += part[static_cast<size_t>(q) * h + i];
+    part[i] = y;   // this thread's own element: read back below by the same thread
+    ss = fmaf(y, y, ss);
+  }
+  const float r = rsqrtf(block_sum(ss, scratch) / static_cast<float>(h) + eps);
+  for (int i = tid; i < h; i += blockDim.x) xr[i] = fmaf(part[i] * r, w[i], row[i]);
+}
+
 template <typename T, typename D>
 static int token_side_launch(float* x, const float* bias, const void* owed, const int* tokens,
                              const void* side, const void* gate, const void* proj, const float* w,
                              float eps, int n, int h, int dim, int vocab, int side_stride, int col0,
-                             hipStream_t s) {
+                             const void* proj_t, hipStream_t s) {
   if (n <= 0) return 0;
+  auto at16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if (proj_t && h % 8 == 0 && dim % 8 == 0 && at16(gate) && at16(proj_t)) {
+    const int chunks = h / 8;
+    const int CC = chunks < 1024 ? chunks : 1024;
+    int JG = 1024 / CC;
+    if (JG > dim) JG = dim;
+    const size_t wide = (static_cast<size_t>(1 + JG) * h + dim) * sizeof(float);
+    if (wide <= 64 * 1024) {
+      hipLaunchKernelGGL((token_side_wide_kernel<T, D>), dim3(n), dim3(1024), wide, s, x, bias,
+                         static_cast<const D*>(owed), tokens, static_cast<const T*>(side),
+                         static_cast<const T*>(gate), static_cast<const T*>(proj_t), w, eps, h, dim, vocab,
+                         side_stride, col0, CC, JG);
+      return kvf_last_error();
+    }
+  }
   const size_t lds = static_cast<size_t>(h + dim) * sizeof(float);
   if (lds > 64 * 1024) return static_cast<int>(hipErrorInvalidValue);
   hipLaunchKernelGGL((token_side_kernel<T, D>), dim3(n), dim3(256), lds, s, x, bias,
@@ -773,18 +911,20 @@ static int token_side_launch(float* x, const float* bias, const void* owed, cons
 #define TOKEN_SIDE_DECL                                                                          \
   float *x, const float *bias, const void *owed, int owed_f32, const int *tokens,               \
       const void *side, const void *gate, const void *proj, const float *w, float eps, int n,   \
-      int h, int dim, int vocab, int side_stride, int col0, hipStream_t s
+      int h, int dim, int vocab, int side_stride, int col0, const void *proj_t, hipStream_t s
+// proj_t (may be null): proj transposed, [dim, h]; with it, rows of a multiple of 8 elements take
+// the kernel of 1,024 threads
 KVF_EXPORT int kvf_token_side_f32(TOKEN_SIDE_DECL) {
   (void)owed_f32;
   return token_side_launch<float, float>(x, bias, owed, tokens, side, gate, proj, w, eps, n, h, dim,
-                                         vocab, side_stride, col0, s);
+                                         vocab, side_stride, col0, proj_t, s);
 }
 KVF_EXPORT int kvf_token_side_bf16(TOKEN_SIDE_DECL) {
   if (owed_f32)
     return token_side_launch<bf16_t, float>(x, bias, owed, tokens, side, gate, proj, w, eps, n, h, dim,
-                                            vocab, side_stride, col0, s);
+                                            vocab, side_stride, col0, proj_t, s);
   return token_side_launch<bf16_t, bf16_t>(x, bias, owed, tokens, side, gate, proj, w, eps, n, h, dim,
-                                           vocab, side_stride, col0, s);
+                                           vocab, side_stride, col0, proj_t, s);
 }
 
 // ----------------------------------------------------------------------------- the same, in pieces

@@ -247,12 +247,14 @@ TOKEN_SIDE_MAX_FLOATS = 16 * 1024   # the row and the gated vector live in 64 KB
 
 def token_side(x: torch.Tensor, tokens: torch.Tensor, side: torch.Tensor, col0: int,
                gate: torch.Tensor, proj: torch.Tensor, weight: torch.Tensor, eps: float,
-               bias: torch.Tensor | None = None, owed: torch.Tensor | None = None) -> None:
+               bias: torch.Tensor | None = None, owed: torch.Tensor | None = None,
+               proj_t: torch.Tensor | None = None) -> None:
     """A per-token input into the fp32 stream: with ``e = side[token, col0 : col0 + dim]``,
     ``y = proj @ (gelu_tanh(gate @ x[m]) * e)`` and ``x[m] += y * rsqrt(mean(y^2) + eps) * weight``.
     ``bias`` (fp32 ``[h]``) and ``owed`` (``[M, h]``, a product still owed to the stream) are added
     to ``x[m]`` first and stay in it.  ``gate [dim, h]``, ``proj [h, dim]`` and ``side`` share a
-    type; ``weight`` is fp32."""
+    type; ``weight`` is fp32.  ``proj_t``: ``proj`` transposed, ``[dim, h]`` contiguous; with it,
+    rows of a multiple of 8 elements take a kernel of 1,024 threads with 16-byte loads."""
     _check(x, "x", F32, (None, None))
     n, h = x.shape
     _check(tokens, "tokens", I32, (None,))
@@ -273,13 +275,16 @@ def token_side(x: torch.Tensor, tokens: torch.Tensor, side: torch.Tensor, col0: 
         _check(owed, "owed", None, (n, h))
         if owed.dtype not in (F32, gate.dtype):
             raise KernelError(f"token_side: owed must be float32 or {gate.dtype}, got {owed.dtype}")
+    if proj_t is not None:
+        _check(proj_t, "proj_t", gate.dtype, (dim, h))
     f = _fn("elementwise", f"kvf_token_side_{_suffix(gate.dtype)}",
-            [c_void_p, c_void_p, c_void_p, c_int] + [c_void_p] * 5 + [c_float] + [c_int] * 6 + [c_void_p])
+            [c_void_p, c_void_p, c_void_p, c_int] + [c_void_p] * 5 + [c_float] + [c_int] * 6 + [c_void_p, c_void_p])
     _ok(f(x.data_ptr(), bias.data_ptr() if bias is not None else None,
           owed.data_ptr() if owed is not None else None,
           1 if owed is not None and owed.dtype == F32 else 0, tokens.data_ptr(), side.data_ptr(),
           gate.data_ptr(), proj.data_ptr(), weight.data_ptr(), float(eps), n, h, dim, side.shape[0],
-          side.shape[1], int(col0), _stream()), "token_side")
+          side.shape[1], int(col0), proj_t.data_ptr() if proj_t is not None else None, _stream()),
+        "token_side")
 
 
 def settle_cast(x: torch.Tensor, bias: torch.Tensor | None = None, owed: torch.Tensor | None = None,

@@ -30,7 +30,7 @@ class TokenSideInput(Part):
         self.prefix, self.hidden, self.dim, self.vocab = prefix, int(hidden), int(dim), int(vocab)
         self.table_name, self.table_cols, self.first_col = table_name, int(table_cols), int(first_col)
         self.eps = float(eps)
-        self.table = self.gate = self.proj = self.weight = None
+        self.table = self.gate = self.proj = self.proj_t = self.weight = None
 
     def weight_specs(self) -> dict[str, WeightSpec]:
         return {self.table_name: WeightSpec((self.vocab, self.table_cols)),
@@ -44,6 +44,8 @@ class TokenSideInput(Part):
         if not (self.table.dtype == self.gate.dtype == self.proj.dtype):
             self.table, self.gate, self.proj = self.table.float(), self.gate.float(), self.proj.float()
         self.weight = tensors[self._name("norm")].float().contiguous()
+        # the projection once more, transposed: what the kernel for few rows reads side by side
+        self.proj_t = self.proj.t().contiguous()
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
         return {"elementwise", "gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())
@@ -52,7 +54,7 @@ class TokenSideInput(Part):
         return sum(t.numel() * t.element_size() for t in (self.gate, self.proj, self.weight) if t is not None)
 
     def held_tensors(self) -> list[torch.Tensor]:
-        return [t for t in (self.table, self.gate, self.proj, self.weight) if t is not None]
+        return [t for t in (self.table, self.gate, self.proj, self.proj_t, self.weight) if t is not None]
 
     # rows up to which one kernel does everything, a workgroup per row with the two small
     # matrices read through the caches; beyond, the two products go to the matrix kernels
@@ -64,7 +66,7 @@ class TokenSideInput(Part):
         owed = step.take_owed(residual)
         if n <= self.FUSED_MAX_ROWS:
             ops.token_side(residual, step.token_ids, self.table, self.first_col, self.gate, self.proj,
-                           self.weight, self.eps, bias=bias, owed=owed)
+                           self.weight, self.eps, bias=bias, owed=owed, proj_t=self.proj_t)
             return
         ws, dt = step.ws, self.gate.dtype
         x = residual

@@ -133,8 +133,12 @@ def test_sigmoid_gate_reads_a_block_of_columns(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("h,dim,extras", [(24, 3, "both"), (96, 8, "none"), (2500, 17, "bias"), (256, 64, "owed")])
-def test_token_side(dtype, h, dim, extras):
+@pytest.mark.parametrize("h,dim,extras", [(24, 3, "both"), (96, 8, "none"), (2500, 17, "bias"), (256, 64, "owed"),
+                                          (2048, 64, "both"), (4096, 128, "bias"), (8200, 8, "none"), (40, 1024, "owed")])
+@pytest.mark.parametrize("transposed", [False, True])
+def test_token_side(dtype, h, dim, extras, transposed):
+    """``transposed``: the projection is also given transposed, which lets rows of a multiple of
+    eight elements take the kernel of 1,024 threads."""
     n, vocab, layers, layer = 6, 11, 3, 1
     x = rand(n, h, seed=1)
     side, gate, proj = (rand(vocab, layers * dim, seed=2).to(dtype), rand(dim, h, seed=3, scale=h ** -0.5).to(dtype),
@@ -145,7 +149,8 @@ def test_token_side(dtype, h, dim, extras):
     tokens = torch.tensor([3, 0, 10, 11, -2, 7], dtype=torch.int32)       # two lie outside the table
     got = x.clone().to(DEV)
     ops().token_side(got, tokens.to(DEV), side.to(DEV), layer * dim, gate.to(DEV), proj.to(DEV), w.to(DEV),
-                     1e-5, bias=None if bias is None else bias.to(DEV), owed=None if owed is None else owed.to(DEV))
+                     1e-5, bias=None if bias is None else bias.to(DEV), owed=None if owed is None else owed.to(DEV),
+                     proj_t=proj.t().contiguous().to(DEV) if transposed else None)
     base = x + (bias if bias is not None else 0.0) + (owed.float() if owed is not None else 0.0)
     known = (tokens >= 0) & (tokens < vocab)
     rows = side.float()[tokens.clamp(0, vocab - 1).long()][:, layer * dim:(layer + 1) * dim]
