@@ -644,11 +644,50 @@ __global__ void gated_act_kernel(const T* __restrict__ gu, const float* __restri
   if (bu) u += bu[i];
   Elem<T>::store(out + idx, act_f(act, g) * u);
 }
+// bf16, paired: a thread takes four neighbouring (gate, up) pairs (16 bytes in, 8 bytes out)
+__global__ void gated_act_pairs4_kernel(const bf16_t* __restrict__ gu, const float* __restrict__ bg,
+                                        const float* __restrict__ bu, bf16_t* __restrict__ out,
+                                        int inter, size_t quads, int act) {
+  const size_t q = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (q >= quads) return;
+  float v[8];
+  load8(gu + q * 8, v);
+  const int i0 = static_cast<int>((q * 4) % inter);   // inter is a multiple of 4: one row
+  uint32_t hh[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float g = v[2 * i], u = v[2 * i + 1];
+    if (bg) g += bg[i0 + i];
+    if (bu) u += bu[i0 + i];
+    float a;
+    if (act == 1) {
+      // tanh(t) = 1 - 2 / (1 + exp(2 t)); exp overflows to +inf for large t, which gives 1
+      const float t = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+      a = 0.5f * g * (2.f - 2.f / (1.f + __expf(2.f * t)));
+    } else {
+      a = g / (1.f + __expf(-g));
+    }
+    hh[i] = f32_to_bf16(a * u);
+  }
+  uint2 packed;
+  packed.x = hh[0] | (hh[1] << 16);
+  packed.y = hh[2] | (hh[3] << 16);
+  *reinterpret_cast<uint2*>(out + q * 4) = packed;
+}
+
 template <typename T>
 static int gated_act_launch(const void* gu, const float* bg, const float* bu, void* out, int m,
                             int inter, int paired, int act, hipStream_t s) {
   const size_t total = static_cast<size_t>(m) * inter;
   if (total == 0) return 0;
+  if (sizeof(T) == 2 && paired && inter % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(out) % 8 == 0) {
+    const size_t quads = total / 4;
+    hipLaunchKernelGGL(gated_act_pairs4_kernel, dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256),
+                       0, s, static_cast<const bf16_t*>(gu), bg, bu, static_cast<bf16_t*>(out), inter, quads,
+                       act);
+    return kvf_last_error();
+  }
   hipLaunchKernelGGL(gated_act_kernel<T>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, s,
                      static_cast<const T*>(gu), bg, bu, static_cast<T*>(out), inter, total, paired, act);
   return kvf_last_error();

@@ -107,9 +107,10 @@ def test_norm_shift_leaves_sequences_without_a_slot_alone():
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("activation", ["gelu_tanh", "silu"])
 @pytest.mark.parametrize("paired,bias", [(True, True), (False, True), (True, False)])
-def test_gated_act(dtype, activation, paired, bias):
-    m, inter = 7, 37
-    gate, up = rand(m, inter, seed=1, scale=2.0).to(dtype), rand(m, inter, seed=2).to(dtype)
+@pytest.mark.parametrize("inter", [37, 72])        # 72: four pairs per thread in bfloat16
+def test_gated_act(dtype, activation, paired, bias, inter):
+    m = 7
+    gate, up = rand(m, inter, seed=1, scale=4.0).to(dtype), rand(m, inter, seed=2).to(dtype)
     bg, bu = (rand(inter, seed=3), rand(inter, seed=4)) if bias else (None, None)
     gu = torch.stack([gate, up], dim=2).reshape(m, 2 * inter) if paired else torch.cat([gate, up], dim=1)
     out = torch.empty(m, inter, dtype=dtype, device=DEV)
