@@ -645,20 +645,23 @@ __global__ void gated_act_kernel(const T* __restrict__ gu, const float* __restri
   Elem<T>::store(out + idx, act_f(act, g) * u);
 }
 // bf16, paired: a thread takes four neighbouring (gate, up) pairs (16 bytes in, 8 bytes out)
+// (the grid's x runs along a row, its y over the rows, so that no index is divided)
 __global__ void gated_act_pairs4_kernel(const bf16_t* __restrict__ gu, const float* __restrict__ bg,
                                         const float* __restrict__ bu, bf16_t* __restrict__ out,
-                                        int inter, size_t quads, int act) {
-  const size_t q = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (q >= quads) return;
+                                        int inter, int rows, int act) {
+  const int i0 = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (i0 >= inter) return;
+  float4 b_g = make_float4(0.f, 0.f, 0.f, 0.f), b_u = b_g;
+  if (bg) b_g = *reinterpret_cast<const float4*>(bg + i0);
+  if (bu) b_u = *reinterpret_cast<const float4*>(bu + i0);
+  const float gb[4] = {b_g.x, b_g.y, b_g.z, b_g.w}, ub[4] = {b_u.x, b_u.y, b_u.z, b_u.w};
+  for (int m = blockIdx.y; m < rows; m += gridDim.y) {
   float v[8];
-  load8(gu + q * 8, v);
-  const int i0 = static_cast<int>((q * 4) % inter);   // inter is a multiple of 4: one row
+  load8(gu + (static_cast<size_t>(m) * inter + i0) * 2, v);
   uint32_t hh[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    float g = v[2 * i], u = v[2 * i + 1];
-    if (bg) g += bg[i0 + i];
-    if (bu) u += bu[i0 + i];
+    const float g = v[2 * i] + gb[i], u = v[2 * i + 1] + ub[i];
     float a;
     if (act == 1) {
       // tanh(t) = 1 - 2 / (1 + exp(2 t)); exp overflows to +inf for large t, which gives 1
@@ -672,7 +675,8 @@ __global__ void gated_act_pairs4_kernel(const bf16_t* __restrict__ gu, const flo
   uint2 packed;
   packed.x = hh[0] | (hh[1] << 16);
   packed.y = hh[2] | (hh[3] << 16);
-  *reinterpret_cast<uint2*>(out + q * 4) = packed;
+  *reinterpret_cast<uint2*>(out + static_cast<size_t>(m) * inter + i0) = packed;
+  }
 }
 
 template <typename T>
@@ -680,12 +684,13 @@ static int gated_act_launch(const void* gu, const float* bg, const float* bu, vo
                             int inter, int paired, int act, hipStream_t s) {
   const size_t total = static_cast<size_t>(m) * inter;
   if (total == 0) return 0;
-  if (sizeof(T) == 2 && paired && inter % 4 == 0 && reinterpret_cast<uintptr_t>(gu) % 16 == 0 &&
-      reinterpret_cast<uintptr_t>(out) % 8 == 0) {
-    const size_t quads = total / 4;
-    hipLaunchKernelGGL(gated_act_pairs4_kernel, dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256),
-                       0, s, static_cast<const bf16_t*>(gu), bg, bu, static_cast<bf16_t*>(out), inter, quads,
-                       act);
+  auto at16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  if (sizeof(T) == 2 && paired && inter % 4 == 0 && at16(gu) && reinterpret_cast<uintptr_t>(out) % 8 == 0 &&
+      at16(bg) && at16(bu)) {
+    const int threads = inter / 4 >= 256 ? 256 : 64;
+    const dim3 grid((inter / 4 + threads - 1) / threads, m < 65535 ? m : 65535);
+    hipLaunchKernelGGL(gated_act_pairs4_kernel, grid, dim3(threads), 0, s, static_cast<const bf16_t*>(gu), bg,
+                       bu, static_cast<bf16_t*>(out), inter, m, act);
     return kvf_last_error();
   }
   hipLaunchKernelGGL(gated_act_kernel<T>, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, s,
