@@ -417,7 +417,16 @@ def shape_c() -> dict:
                        window=1000, keep_first=4, side_dim=64, max_positions=400, share_every=1)
 
 
-SHAPE = {"a": shape_a, "b": shape_b, "c": shape_c}
+def shape_d() -> dict:
+    """Layers wide enough for what serving a real model takes: tiled weights, a down projection
+    deep and narrow enough to be cut in two halves of K (one half stays owed to the stream until
+    the per-layer input takes it), gate/up wide enough for two groups of columns a wave, the
+    kernel of 1,024 threads for the per-layer input."""
+    return make_config(vocab=1000, width=256, layers=2, heads=4, kv_heads=2, dim=64, ff=4096,
+                       window=50, keep_first=3, side_dim=24, max_positions=400, share_every=2)
+
+
+SHAPE = {"a": shape_a, "b": shape_b, "c": shape_c, "d": shape_d}
 
 
 def liven(folder: str) -> None:
