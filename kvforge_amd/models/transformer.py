@@ -9,7 +9,7 @@ import torch
 from kvforge_amd import registry
 from kvforge_amd.cache.manager import CacheGroup
 from kvforge_amd.kernels import library
-from kvforge_amd.parts.base import Block, CacheSpec, LayerState, ModelSpec, Positions, StateSpec
+from kvforge_amd.parts.base import Block, CacheSpec, LayerState, ModelSpec, StateSpec
 from kvforge_amd.weights.loader import load_model_weights
 
 
@@ -144,20 +144,21 @@ class Transformer:
     def can_pick(self, rows: int) -> bool:
         """Whether a decode step of ``rows`` sequences can end in the head's greedy pick
         (``forward(step, tail=...)``): the parts say so themselves.  The embedding names a bf16
-        table that holds its outputs (``Embedding.pick_table``), no position encoding touches
-        the embedding output, and the head takes so many rows (``Head.can_pick``)."""
+        table that holds its outputs (``Embedding.pick_table``) and the head takes so many rows
+        (``Head.can_pick``).  Position encodings that act on the embedding output are no
+        hindrance: the pick leaves the table's rows in the stream and moves the positions on,
+        and ``forward`` applies the encodings to a stream that is handed to it (``embedded``)
+        as it does to one it fills itself."""
         spec = self.spec
-        untouched = all(type(p).on_embedding is Positions.on_embedding for p in spec.positions)
-        return (self.dtype == torch.bfloat16 and untouched
+        return (self.dtype == torch.bfloat16
                 and spec.embedding.pick_table() is not None and spec.head.can_pick(rows))
 
     def embed(self, step) -> torch.Tensor:
-        """The step's residual stream, filled from the embedding."""
+        """The step's residual stream, filled from the embedding table alone (what ``forward``
+        expects to find with ``embedded``; position encodings on it are ``forward``'s)."""
         spec = self.spec
         residual = step.ws.buf("residual", (step.n_tokens, spec.embedding.hidden), torch.float32)
         spec.embedding.forward(step.token_ids, residual)
-        for p in spec.positions:
-            p.on_embedding(residual, step)
         return residual
 
     def forward(self, step, tail=None, embedded: bool = False) -> torch.Tensor | None:
@@ -176,6 +177,8 @@ class Transformer:
             residual = step.ws.buf("residual", (step.n_tokens, hidden), torch.float32)
         else:
             residual = self.embed(step)
+        for p in spec.positions:
+            p.on_embedding(residual, step)
         for call, ls in zip(self.order, self.layer_states):
             spec.blocks[call.layer].forward(residual, step, ls)
         r = step.n_logits

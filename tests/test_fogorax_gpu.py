@@ -575,6 +575,8 @@ def test_the_stream_after_every_layer(tmp_path_factory):
     model = runner.model
     with torch.inference_mode():
         residual = model.embed(step)
+        for p in model.spec.positions:
+            p.on_embedding(residual, step)
         for i, (call, ls) in enumerate(zip(model.order, model.layer_states)):
             model.spec.blocks[call.layer].forward(residual, step, ls)
             step.settle()
