@@ -298,7 +298,7 @@ def give_back_hidden_pages(paged, seq_lens, q_lens, bs, window, keep):
             paged.table[s, b] = -1
 
 
-MASKS = [(11, 3), (40, 4), (64, 33), (5, 0), (7, 70), (33, 1)]
+MASKS = [(11, 3), (40, 4), (64, 33), (5, 0), (7, 70), (33, 1), (1, 2), (2048, 4)]
 SHAPES = [(4, 2, 16, 4), (6, 2, 32, 8), (3, 1, 48, 16), (8, 2, 64, 16), (32, 8, 64, 16), (4, 1, 128, 32), (5, 5, 80, 24)]
 
 
@@ -673,6 +673,27 @@ def test_greedy_generation_through_the_engine(tmp_path_factory, name, dtype):
     assert engine.cache.slots.num_free == 3 and engine.cache.num_free_blocks == 48
     if engine.runner.use_graphs:
         assert engine.runner.num_graph_replays > 0
+
+
+def test_a_request_that_loses_its_pages_and_slot_is_read_again_from_its_first_token(tmp_path_factory):
+    """Nothing is given back behind this shape's window, so three requests outgrow the pool:
+    the scheduler takes one's pages and state slot away and feeds it again later, prompt and
+    generated tokens, into a slot and pages that others have used."""
+    folder, cfg, w = model_folder(tmp_path_factory, "c", torch.float32)
+    engine = kvforge_amd.InferenceEngine.from_folder(
+        folder, kvforge_amd.EngineConfig(
+            cache=kvforge_amd.CacheConfig(block_size=8, num_blocks=20, watermark=0.0), dtype=torch.float32,
+            scheduler=kvforge_amd.SchedulerConfig(max_num_seqs=3, max_num_batched_tokens=32, max_model_len=128)))
+    prompts = list(prompts_for(cfg, [30, 26, 33], 10).values())
+    outs = engine.generate(prompts, kvforge_amd.SamplingParams(max_tokens=40, temperature=0.0, ignore_eos=True))
+    assert engine.scheduler.num_preemptions > 0
+    for p, o in zip(prompts, outs):
+        assert len(o.output_token_ids) == 40
+        logits = plain.forward(cfg, w, p + o.output_token_ids)
+        for i, tok in enumerate(o.output_token_ids):
+            row = logits[len(p) - 1 + i]
+            assert float(row.max() - row[tok]) <= 1e-3 * float(row.std()), (i, tok)
+    assert engine.cache.slots.num_free == 3 and engine.cache.num_free_blocks == 20
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
