@@ -675,6 +675,87 @@ def test_greedy_generation_through_the_engine(tmp_path_factory, name, dtype):
         assert engine.runner.num_graph_replays > 0
 
 
+def random_shape(seed: int) -> dict:
+    """A model whose every size, count, constant and layer order is drawn: widths that are no
+    multiple of 8, head sizes that are no multiple of 16, query/key and value sizes apart, any
+    group size, windows from one key up, kept keys from none up, layers that read any earlier
+    layer with keys of its own (each reader with a mask of its own), layers without a
+    feed-forward, with and without the per-layer input."""
+    import random
+    rng = random.Random(seed)
+    kv_heads = rng.choice([1, 2, 3])
+    heads = kv_heads * rng.choice([1, 2, 3, 4])
+    dim, vdim = rng.choice([8, 16, 20, 32, 48, 64, 72]), rng.choice([8, 16, 24, 32, 40, 64, 80])
+    width = rng.choice([24, 36, 50, 64, 88, 100, 128, 200])
+    n = rng.randint(1, 6)
+    layers, owners = [], []
+    for i in range(n):
+        mixer = {"dim": dim, "heads": heads, "kv_heads": kv_heads, "vdim": vdim,
+                 "mask": {"keep_first": rng.choice([0, 0, 1, 2, 5, 9, 17]), "size": rng.choice([1, 2, 7, 16, 25, 40, 64, 300])},
+                 "scale": rng.choice([0.05, 0.125, 0.3, dim ** -0.5])}
+        if owners and rng.random() < 0.5:
+            mixer["kv_from"] = rng.choice(owners)
+        else:
+            owners.append(i)
+        mlp = None if rng.random() < 0.2 else {"ff": rng.choice([8, 31, 64, 130, 256]), "kind": "dense"}
+        layers.append({"mixer": mixer, "mlp": mlp, "type": "attention"})
+    side = rng.choice([0, 1, 6, 8, 16, 40])
+    return {"architecture": "Fogorax", "layers": layers, "max_positions": 256,
+            "norm": {"eps": rng.choice([1e-6, 1e-5, 1e-3, 0.1])},
+            "token_side": {"dim": side} if side else None,
+            "vocab": rng.choice([17, 64, 100, 257, 512]), "width": width}
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", range(12))
+def test_models_drawn_at_random(tmp_path, seed, dtype):
+    """Whole, token by token, in portions and in a batch with pages and slots used again."""
+    cfg = random_shape(seed)
+    folder = str(tmp_path / "model")
+    kvforge_amd.write_random_model(folder, cfg, seed=seed, dtype=NAME[dtype])
+    liven(folder)
+    w = load_file(os.path.join(folder, "model.safetensors"))
+    bs = [4, 8, 16, 24][seed % 4]
+    seqs = prompts_for(cfg, [90, 41, 2, 64, 33], seed)
+    runner = make_runner(folder, dtype, block_size=bs, num_blocks=-(-260 // bs), seqs=3)
+    plan = ([[("r0", 0, 90)]] + [[("r1", i, i + 1)] for i in range(41)] + in_portions("r3", 64, (5, 2, 17, 3))
+            + [[("r0", 0, 40), ("r2", 0, 1)], [("r2", 1, 2), ("r0", 40, 41), ("r4", 0, 20)],
+               [("r0", 41, 90), ("r4", 20, 21), ("r1", 0, 30)], [("r4", 21, 33), ("r1", 30, 41)]])
+    got: dict = {}
+    for r, v in replay_all(runner, seqs, plan).items():
+        got[r] = v
+    for r, t in seqs.items():
+        for k, logits in enumerate(got[r]):
+            check(logits, cfg, w, t, dtype, f"seed {seed}, {r}, pass {k}: {cfg}")
+    assert runner.cache.slots.num_free == 3 and runner.cache.num_free_blocks == -(-260 // bs)
+
+
+def replay_all(runner, seqs, plan) -> dict:
+    """Like ``replay`` for a plan that reads requests more than once: a list of whole-sequence
+    logits per request, one per time it was read to its end."""
+    out = {r: [] for r in seqs}
+    part = {r: [] for r in seqs}
+    cache = runner.cache
+    for step in plan:
+        entries = []
+        for rid, a, b in step:
+            if not cache.has_request(rid):
+                cache.allocate(rid, 0)
+            cache.append_slots(rid, b, a)
+            entries.append(StepEntry(rid, seqs[rid][a:b], a, "all"))
+        logits = runner.step(entries).cpu()
+        off = 0
+        for rid, a, b in step:
+            part[rid].append(logits[off:off + b - a].clone())
+            off += b - a
+            cache.release_behind(rid, b)
+            if b == len(seqs[rid]):
+                cache.free(rid)
+                out[rid].append(torch.cat(part[rid]))
+                part[rid] = []
+    return out
+
+
 def test_a_request_that_loses_its_pages_and_slot_is_read_again_from_its_first_token(tmp_path_factory):
     """Nothing is given back behind this shape's window, so three requests outgrow the pool:
     the scheduler takes one's pages and state slot away and feeds it again later, prompt and
