@@ -92,6 +92,9 @@ class ParallelBlock(Block):
         super().load(tensors)
         if self.shift_name is not None:
             self.mu = tensors[self.shift_name].float().contiguous()
+            # the fused kernel multiplies by fp32 vectors
+            if self.norm.weight.dtype != torch.float32:
+                self.norm.weight = self.norm.weight.float()
 
     def kernel_modules(self, dtype) -> set[str]:
         return super().kernel_modules(dtype) | {"elementwise"}
@@ -102,21 +105,14 @@ class ParallelBlock(Block):
     def num_bytes(self) -> int:
         return super().num_bytes() + (4 * self.mu.numel() if self.mu is not None else 0)
 
-    @property
-    def replayable(self) -> bool:
-        return all(p.replayable for p in self.parts())
-
     def forward(self, residual, step, layer: LayerState) -> None:
         shape = tuple(residual.shape)
         h = step.ws.buf("parallel_normed", shape, step.act_dtype)
         if self.mu is not None:
             step.settle()
             hs = step.ws.buf("parallel_shifted", shape, step.act_dtype)
-            w = self.norm.weight
-            if w.dtype != torch.float32:
-                w = self.norm.weight = w.float()
-            ops.norm_shift(residual, w, self.mu, layer.state, step.slot_ids, step.seq_of_token,
-                           step.cu_q, step.positions, self.norm.eps, h, hs)
+            ops.norm_shift(residual, self.norm.weight, self.mu, layer.state, step.slot_ids,
+                           step.seq_of_token, step.cu_q, step.positions, self.norm.eps, h, hs)
         else:
             self.norm.forward(residual, h, add=step.take_owed(residual))
             hs = h

@@ -675,6 +675,48 @@ def test_greedy_generation_through_the_engine(tmp_path_factory, name, dtype):
         assert engine.runner.num_graph_replays > 0
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_parallel_block_without_shift_or_anything_behind_it(dtype):
+    """The block as another design would use it: a norm with a weight vector, plain attention
+    (no gate, no window) and a silu feed-forward without biases side by side."""
+    from kvforge_amd.engine.batch import MetaBuffers, Step, Workspace, fill_step
+    from kvforge_amd.cache.manager import CacheGroup, CacheManager
+    from kvforge_amd.parts import GatedFeedForward, LayerState, PagedAttention, ParallelBlock, RMSNorm
+
+    h, H, KV, d, ff, n, bs = 48, 4, 2, 16, 40, 21, 8
+    block = ParallelBlock(RMSNorm("n", h, 1e-5), PagedAttention("a", h, H, KV, d, None, scale=0.2),
+                          GatedFeedForward("f", h, ff), h)
+    assert block.state_spec is None
+    names = {k: rand(*v.shape, seed=i, scale=0.3) + (1.0 if v.init == "norm" else 0.0)
+             for i, (k, v) in enumerate(sorted(block.weight_specs().items()))}
+    block.load({k: t.to(dtype).to(DEV) for k, t in names.items()})
+    block.seal()
+    w = {k: t.to(dtype).float() for k, t in names.items()}
+    x = rand(n, h, seed=50)
+    cache = CacheManager(bs, [CacheGroup((0,), block.mixer.cache_spec.pages)], 8)
+    cache.allocate("s", 0)
+    layer = LayerState(group=0, pages={"k": torch.zeros(8, KV, bs, d, dtype=dtype, device=DEV),
+                                       "v": torch.zeros(8, KV, d, bs, dtype=dtype, device=DEV)})
+    meta, ws, got = MetaBuffers(64, 4, [8], DEV), Workspace(DEV), []
+    for a, b in ((0, 13), (13, 14), (14, 21)):
+        cache.append_slots("s", b, a)
+        step = Step()
+        step.ws, step.act_dtype, step.device = ws, dtype, DEV
+        fill_step(step, meta, [StepEntry("s", list(range(a, b)), a, "all")], cache.block_table, lambda r: -1, bs)
+        res = x[a:b].clone().to(DEV)
+        block.forward(res, step, layer)
+        step.settle()
+        got.append(res.cpu())
+    hn = plain.rms(x, 1e-5) * w["n.weight"]
+    q, k, v = (hn @ w[f"a.{m}_proj.weight"].T for m in "qkv")
+    o = plain.masked_attention(q.view(n, H, d), k.view(n, KV, d), v.view(n, KV, d), 0.2,
+                               plain.window_mask(n, n, 0)).reshape(n, H * d)
+    g = hn @ w["f.gate_proj.weight"].T
+    want = x + o @ w["a.o_proj.weight"].T + (g * torch.sigmoid(g) * (hn @ w["f.up_proj.weight"].T)) @ w["f.down_proj.weight"].T
+    torch.testing.assert_close(torch.cat(got), want, **(dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32
+                                                         else dict(atol=6e-2, rtol=6e-2)))
+
+
 def random_shape(seed: int) -> dict:
     """A model whose every size, count, constant and layer order is drawn: widths that are no
     multiple of 8, head sizes that are no multiple of 16, query/key and value sizes apart, any
