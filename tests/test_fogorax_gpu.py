@@ -52,7 +52,7 @@ def test_add_positions():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("h", [24, 200, 1031])
+@pytest.mark.parametrize("h", [24, 200, 1031, 4100, 9001])
 def test_norm_shift_over_runs_and_steps(dtype, h):
     """Three sequences in two steps; the second step continues two of them from their state
     slots and starts a new one in the slot the third gave back, which still holds its state."""
