@@ -154,6 +154,8 @@ def add_rows(x: torch.Tensor, delta: torch.Tensor) -> None:
     _ok(f(x.data_ptr(), delta.data_ptr(), x.shape[0], x.shape[1], _stream()), "add_rows")
 
 
+# ------------------------------------------------------------------------------ learned positions,
+# norm + token shift, gated activations, output gate, per-token side input
 def add_positions(x: torch.Tensor, table: torch.Tensor, positions: torch.Tensor) -> None:
     """``x[n] += table[positions[n]]`` for the fp32 stream ``x``: a learned vector per position."""
     _check(x, "x", F32, (None, None))
