@@ -46,7 +46,8 @@ class WindowMask:
 @dataclass(frozen=True)
 class AttentionMixerConfig:
     """``kv_from``: the layer whose keys and values this layer reads instead of projecting its
-    own (``None``: its own)."""
+    own (``None``: its own).  A file may leave out ``kv_heads`` (then as many as ``heads``) and
+    ``vdim`` (then ``dim``)."""
 
     heads: int
     kv_heads: int
@@ -58,7 +59,8 @@ class AttentionMixerConfig:
 
     @classmethod
     def from_dict(cls, d: dict[str, Any], where: str) -> "AttentionMixerConfig":
-        heads, kv_heads = _positive(d, "heads", where), _positive(d, "kv_heads", where)
+        heads = _positive(d, "heads", where)
+        kv_heads = _positive(d, "kv_heads", where) if d.get("kv_heads") is not None else heads
         if heads % kv_heads:
             raise ConfigError(f"{where}: heads ({heads}) must be a multiple of kv_heads ({kv_heads})")
         scale = float(_require(d, "scale"))
@@ -67,8 +69,9 @@ class AttentionMixerConfig:
         kv_from = d.get("kv_from")
         if kv_from is not None and (not isinstance(kv_from, int) or kv_from < 0):
             raise ConfigError(f"{where}: 'kv_from' must name a layer, got {kv_from!r}")
-        return cls(heads, kv_heads, _positive(d, "dim", where), _positive(d, "vdim", where), scale,
-                   WindowMask.from_dict(_require(d, "mask"), where), kv_from)
+        dim = _positive(d, "dim", where)
+        vdim = _positive(d, "vdim", where) if d.get("vdim") is not None else dim
+        return cls(heads, kv_heads, dim, vdim, scale, WindowMask.from_dict(_require(d, "mask"), where), kv_from)
 
     def to_dict(self) -> dict[str, Any]:
         out: dict[str, Any] = {"dim": self.dim, "heads": self.heads}

@@ -44,6 +44,12 @@ def test_config_round_trip_and_registry_key():
     assert isinstance(registry.config_from_dict(alt), FogoraxConfig)
     with pytest.raises(kvforge_amd.ConfigError):
         registry.config_from_dict({"vocab": 5})
+    # kv_heads and vdim may be left out
+    short = copy.deepcopy(d)
+    for i in (1, 3):                  # layer 3 reads layer 1's keys: the two agree again
+        del short["layers"][i]["mixer"]["kv_heads"], short["layers"][i]["mixer"]["vdim"]
+    m = registry.config_from_dict(short).layers[1].mixer
+    assert (m.kv_heads, m.vdim) == (m.heads, m.dim)
 
 
 @pytest.mark.parametrize("change,needle", [
