@@ -3,8 +3,9 @@ from kvforge_amd.config.engine import (CacheConfig, EngineConfig, SchedulerConfi
 from kvforge_amd.config.model import (ConfigError, LlamaConfig, ModelConfig, RopeScaling,
                                       read_config_json)
 from kvforge_amd.config.fogorax import FogoraxConfig
+from kvforge_amd.config.rudorax import RudoraxConfig
 from kvforge_amd.config.presets import PRESETS, preset_dict
 
 __all__ = ["CacheConfig", "EngineConfig", "SchedulerConfig", "SchedulingPolicy", "parse_dtype",
-           "DTYPES", "ConfigError", "FogoraxConfig", "LlamaConfig", "ModelConfig", "RopeScaling",
+           "DTYPES", "ConfigError", "FogoraxConfig", "RudoraxConfig", "LlamaConfig", "ModelConfig", "RopeScaling",
            "read_config_json", "PRESETS", "preset_dict"]

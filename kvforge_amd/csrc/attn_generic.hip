@@ -29,6 +29,7 @@ struct AttnArgs {
   int keep;  // with a window: the first `keep` keys of a sequence stay visible
   float scale;
   const float* slopes;  // null, or one number per q head: slopes[h] * (key - query position) is added to a score
+  const float* sinks;   // null, or one number per q head: exp(sinks[h]) joins the softmax's denominator (a key without a value)
 };
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -258,6 +259,7 @@ __global__ __launch_bounds__(256) void attn_mfma32_kernel(
   }
   if (!row_ok) return;
   T* o = out + static_cast<size_t>(q0 + tok) * a.o_stride + head * D + 4 * g4;
+  if (a.sinks && l_run > 0.f) l_run += expf(a.sinks[head] - m_run);
   const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
 #pragma unroll
   for (int t = 0; t < DT; ++t)
@@ -299,6 +301,7 @@ struct DecodeArgs {
   int keep;  // as in AttnArgs
   float scale;
   const float* slopes;  // as in AttnArgs
+  const float* sinks;   // as in AttnArgs
 };
 
 // GT: heads of the group handled together (a power of two, at most 8; a larger group is taken
@@ -480,6 +483,7 @@ __global__ __launch_bounds__(DEC_WAVES * KVF_WAVE) void attn_decode_kernel(
       }
     }
     const int head = kvh * G + g0 + g;
+    if (a.splits == 1 && a.sinks && l > 0.f) l += expf(a.sinks[head] - m);
     if (a.splits == 1) {
       // a sequence without context (padding of a captured batch) gets zeros, as the merge
       // kernel gives it: no row of the output keeps what an earlier step left there
@@ -523,6 +527,7 @@ __global__ __launch_bounds__(KVF_WAVE) void attn_decode_merge_kernel(
         l += part_ml[2 * (p0 + c) + 1] * f;
         o += part_acc[(p0 + c) * a.d + e] * f;
       }
+      if (a.sinks && l > 0.f) l += expf(a.sinks[head] - m);
     }
     Elem<T>::store(out + static_cast<size_t>(token) * a.o_stride + head * a.d + e, l > 0.f ? o / l : 0.f);
   }
@@ -577,13 +582,13 @@ KVF_EXPORT int kvf_attn_generic_decode(int dtype, const void* q, const void* k_p
                                        int H, int KV, int d, int block_size, int num_blocks,
                                        int table_stride, int q_stride, int o_stride, int window,
                                        int keep, int n_seqs, int splits, float scale,
-                                       const float* slopes, hipStream_t s) {
+                                       const float* slopes, const float* sinks, hipStream_t s) {
   if (num_seqs <= 0) return 0;
   if (keep < 0 || d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || splits < 1 ||
       (splits > 1 && (!part_acc || !part_ml)) || block_size <= 0)
     return static_cast<int>(hipErrorInvalidValue);
   DecodeArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
-               splits, keep, scale, slopes};
+               splits, keep, scale, slopes, sinks};
   if (dtype == 0)
     return launch_decode<float>(q, k_pages, v_pages, block_table, seq_ids, cu_q, ctx_lens, out,
                                 part_acc, part_ml, num_seqs, a, s);
@@ -601,12 +606,12 @@ KVF_EXPORT int kvf_attn_generic(int dtype, const void* q, const void* k_pages, c
                                 const int* work, int num_work, void* out, int H, int KV, int d,
                                 int block_size, int num_blocks, int table_stride, int q_stride,
                                 int o_stride, int window, int keep, int n_seqs, float scale,
-                                const float* slopes, hipStream_t s) {
+                                const float* slopes, const float* sinks, hipStream_t s) {
   if (keep < 0 || d % 16 != 0 || d > 256 || d <= 0 || KV <= 0 || H % KV != 0 || !work || block_size <= 0 ||
       q_stride % 4 != 0 || o_stride % 4 != 0)
     return static_cast<int>(hipErrorInvalidValue);
   AttnArgs a{H, KV, d, block_size, num_blocks, table_stride, q_stride, o_stride, window, n_seqs,
-             keep, scale, slopes};
+             keep, scale, slopes, sinks};
   if (dtype == 0)
     return launch<float>(q, k_pages, v_pages, block_table, cu_q, ctx_lens, work, num_work, out, a, s);
   if (dtype == 1)

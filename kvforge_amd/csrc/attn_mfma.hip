@@ -78,6 +78,9 @@ struct MArgs {
   // output is multiplied by sigmoid(gate[token, h * d + e]) as it is stored
   const bf16_t* gate;
   int gate_stride;
+  // null, or one number per q head: exp(sinks[h]) joins the softmax's denominator, a key without
+  // a value whose score is not scaled
+  const float* sinks;
 };
 
 // A walk over the blocks of 32 keys that a range of rows sees: blocks counted from `first` up to
@@ -578,8 +581,9 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
 
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    const float l = row_sum(l_run[rt]);
+    float l = row_sum(l_run[rt]);
     if (!rows.ok[rt]) continue;
+    if (a.sinks && l > 0.f) l += exp2f(fmaf(a.sinks[rows.head[rt]], LOG2E, -m_ref[rt]));
     const float inv = l > 0.f ? 1.f / l : 0.f;
     bf16_t* o = out + static_cast<size_t>(q0 + rows.tok[rt]) * a.o_stride + rows.head[rt] * D + 4 * kg;
     const bf16_t* g = a.gate ? a.gate + static_cast<size_t>(q0 + rows.tok[rt]) * a.gate_stride + rows.head[rt] * D + 4 * kg
@@ -761,6 +765,7 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
     part_ml[slot * 2] = mm;  // in log2 units
     part_ml[slot * 2 + 1] = ll;
   }
+  if (a.splits == 1 && a.sinks && ll > 0.f) ll += exp2f(fmaf(a.sinks[head], LOG2E, -mm));
   const float inv = ll > 0.f ? 1.f / ll : 0.f;
   for (int t = wave; t < DT; t += NW) {  // wave w finishes element tiles w, w + NW, ...
     f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -786,7 +791,7 @@ __global__ __launch_bounds__(64) void attn_split_combine_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml,
     const int* __restrict__ seq_ids, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
     bf16_t* __restrict__ out, int H, int D, int splits, int o_stride, int n_seqs,
-    const bf16_t* __restrict__ gate, int gate_stride) {
+    const bf16_t* __restrict__ gate, int gate_stride, const float* __restrict__ sinks) {
   const int seq = seq_ids ? seq_ids[blockIdx.x] : static_cast<int>(blockIdx.x);
   if (seq < 0 || seq >= n_seqs) return;
   const int head = blockIdx.y, lane = threadIdx.x;
@@ -805,7 +810,8 @@ __global__ __launch_bounds__(64) void attn_split_combine_kernel(
   const int tok = cu_q ? cu_q[seq] : seq;
   const float mm = wave_max(m);
   const float c = m == -INFINITY ? 0.f : exp2f(m - mm);
-  const float ll = wave_sum(l * c);
+  float ll = wave_sum(l * c);
+  if (sinks && ll > 0.f) ll += exp2f(fmaf(sinks[head], LOG2E, -mm));
   const float inv = ll > 0.f ? 1.f / ll : 0.f;
   for (int e = lane; e < D; e += KVF_WAVE) {
     float v = 0.f;
@@ -959,7 +965,7 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
                                      const int* work, int num_work, int rows_per_item, void* out, int H, int KV, int d,
                                      int bs, int nb, int table_stride, int q_stride, int o_stride,
                                      int window, int keep, int n_seqs, float scale, const float* slopes,
-                                     const void* gate, int gate_stride, hipStream_t s) {
+                                     const void* gate, int gate_stride, const float* sinks, hipStream_t s) {
   if (num_work <= 0) return 0;
   if (keep < 0 || (gate && (gate_stride % 4 != 0 || gate_stride < H * d || reinterpret_cast<uintptr_t>(gate) % 8 != 0)))
     return static_cast<int>(hipErrorInvalidValue);
@@ -972,7 +978,7 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
   // of one head and finds them in its own L2 after the first workgroup has brought them in.
   const int kv_fastest = num_work <= 65535 ? 1 : 0;
   const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, 1, keep, kv_fastest, scale, magic_of(bs), slopes,
-                static_cast<const bf16_t*>(gate), gate_stride};
+                static_cast<const bf16_t*>(gate), gate_stride, sinks};
   const dim3 grid = kv_fastest ? dim3(KV, num_work) : dim3(num_work, KV);
   switch (d / 16) {
 #define GO(DT) \
@@ -992,7 +998,7 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
                                     int num_seqs, int H, int KV, int d, int bs, int nb,
                                     int table_stride, int q_stride, int o_stride, int window,
                                     int keep, int n_seqs, int splits, float scale, const float* slopes,
-                                    const void* gate, int gate_stride, hipStream_t s) {
+                                    const void* gate, int gate_stride, const float* sinks, hipStream_t s) {
   if (num_seqs <= 0) return 0;
   if (keep < 0 || (gate && (gate_stride % 4 != 0 || gate_stride < H * d || reinterpret_cast<uintptr_t>(gate) % 8 != 0)))
     return static_cast<int>(hipErrorInvalidValue);
@@ -1000,7 +1006,7 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
       splits > KVF_WAVE || (splits > 1 && (!part_acc || !part_ml)))
     return static_cast<int>(hipErrorInvalidValue);
   const MArgs a{H, KV, d, bs, nb, table_stride, q_stride, o_stride, window, n_seqs, splits, keep, 0, scale, magic_of(bs), slopes,
-                static_cast<const bf16_t*>(gate), gate_stride};
+                static_cast<const bf16_t*>(gate), gate_stride, sinks};
   const int G = H / KV, chunks = (G + 15) / 16;
   if (num_seqs > 65535) return static_cast<int>(hipErrorInvalidValue);
   const dim3 grid(KV * chunks, num_seqs, splits);
@@ -1017,6 +1023,6 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
   if (err || splits == 1) return err;
   hipLaunchKernelGGL(attn_split_combine_kernel, dim3(num_seqs, H), dim3(64), 0, s, part_acc,
                      part_ml, seq_ids, cu_q, ctx_lens, static_cast<bf16_t*>(out), H, d, splits,
-                     o_stride, n_seqs, static_cast<const bf16_t*>(gate), gate_stride);
+                     o_stride, n_seqs, static_cast<const bf16_t*>(gate), gate_stride, sinks);
   return kvf_last_error();
 }

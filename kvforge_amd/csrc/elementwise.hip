@@ -3,10 +3,11 @@
 #include "common.h"
 
 // ----------------------------------------------------------------------------- embedding
-// out[n, :] = table[ids[n], :] widened to fp32.  An id outside [0, vocab) writes zeros.
+// out[n, :] = table[ids[n], :] widened to fp32, times `scale` (an fp32 multiply; 1 changes
+// nothing).  An id outside [0, vocab) writes zeros.
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                             float* __restrict__ out, int h, int vocab) {
+                             float* __restrict__ out, int h, int vocab, float scale) {
   const int n = blockIdx.x;
   const int id = ids[n];
   float* o = out + static_cast<size_t>(n) * h;
@@ -15,21 +16,21 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
     return;
   }
   const T* row = table + static_cast<size_t>(id) * h;
-  for (int i = threadIdx.x; i < h; i += blockDim.x) o[i] = Elem<T>::load(row + i);
+  for (int i = threadIdx.x; i < h; i += blockDim.x) o[i] = Elem<T>::load(row + i) * scale;
 }
 
 template <typename T>
 static int embed_launch(const int* ids, const void* table, float* out, int n, int h, int vocab,
-                        hipStream_t s) {
+                        float scale, hipStream_t s) {
   if (n <= 0) return 0;
   hipLaunchKernelGGL(embed_kernel<T>, dim3(n), dim3(256), 0, s, ids, static_cast<const T*>(table),
-                     out, h, vocab);
+                     out, h, vocab, scale);
   return kvf_last_error();
 }
-KVF_EXPORT int kvf_embed_f32(const int* ids, const void* t, float* o, int n, int h, int v,
-                             hipStream_t s) { return embed_launch<float>(ids, t, o, n, h, v, s); }
-KVF_EXPORT int kvf_embed_bf16(const int* ids, const void* t, float* o, int n, int h, int v,
-                              hipStream_t s) { return embed_launch<bf16_t>(ids, t, o, n, h, v, s); }
+KVF_EXPORT int kvf_embed_f32(const int* ids, const void* t, float* o, int n, int h, int v, float scale,
+                             hipStream_t s) { return embed_launch<float>(ids, t, o, n, h, v, scale, s); }
+KVF_EXPORT int kvf_embed_bf16(const int* ids, const void* t, float* o, int n, int h, int v, float scale,
+                              hipStream_t s) { return embed_launch<bf16_t>(ids, t, o, n, h, v, scale, s); }
 
 // ----------------------------------------------------------------------------- RMS norm
 // y = x * rsqrt(mean(x^2) + eps) * w, all in fp32, rounded once to T on store.
@@ -473,6 +474,118 @@ KVF_EXPORT int kvf_rope_kvwrite_f32(ROPE_ARGS_DECL) {
 KVF_EXPORT int kvf_rope_kvwrite_bf16(ROPE_ARGS_DECL) {
   return rope_launch<bf16_t>(qkv, positions, seq_of_token, cos_t, sin_t, block_table, k_pages,
                              v_pages, n, ROPE_ARGS_PACK, s);
+}
+
+// The same with a norm per head in front of the rotation: every q head and every k head is
+// divided by the root mean square of its first `dk` elements (eps inside the root) and
+// multiplied by a weight vector of dk numbers that all q heads (qw) or all k heads (kw) share,
+// all in fp32 from the projected row; then rotated and stored as above, one rounding.  Elements
+// dk..d-1 of a head (padding of the kernels' head size) are zero and stay zero.  A workgroup
+// takes a token, its waves take the heads in turn; a lane holds the pairs lane and lane + 64.
+template <typename T>
+__global__ __launch_bounds__(256) void qknorm_rope_kvwrite_kernel(
+    T* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ block_table, T* __restrict__ k_pages, T* __restrict__ v_pages,
+    const float* __restrict__ qw, const float* __restrict__ kw, int dk, float eps, RopeArgs a) {
+  const int n = blockIdx.x;
+  const int p = positions[n];
+  const int half = a.rot / 2;
+  T* row = qkv + static_cast<size_t>(n) * a.row_len;
+  const bool pos_ok = p >= 0 && p < a.table_len;
+  const float* cs = cos_t ? cos_t + static_cast<size_t>(pos_ok ? p : 0) * half : nullptr;
+  const float* sn = sin_t ? sin_t + static_cast<size_t>(pos_ok ? p : 0) * half : nullptr;
+  int page = -1, off = 0;
+  if (a.write_kv && pos_ok) {
+    const int seq = seq_of_token[n];
+    const int blk = p / a.block_size;
+    if (seq >= 0 && seq < a.n_seqs && blk < a.table_stride) {
+      page = block_table[static_cast<size_t>(seq) * a.table_stride + blk];
+      if (page >= a.num_blocks) page = -1;
+      off = p - blk * a.block_size;
+    }
+  }
+  const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE, waves = blockDim.x / KVF_WAVE;
+  const int heads = a.H + (a.write_kv ? a.KV : 0);
+  for (int hh = wave; hh < heads; hh += waves) {
+    const bool is_k = hh >= a.H;
+    if (is_k && page < 0) continue;
+    T* x = row + hh * a.d;
+    const float* w = is_k ? kw : qw;
+    float u[2], v[2], ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int e = 2 * (lane + KVF_WAVE * j);
+      u[j] = e < dk ? Elem<T>::load(x + e) : 0.f;
+      v[j] = e + 1 < dk ? Elem<T>::load(x + e + 1) : 0.f;
+      ss = fmaf(u[j], u[j], fmaf(v[j], v[j], ss));
+    }
+    const float r = 1.f / sqrtf(wave_sum(ss) / static_cast<float>(dk) + eps);
+    T* dst = is_k ? k_pages + ((static_cast<size_t>(page) * a.KV + (hh - a.H)) * a.block_size + off) * a.d : x;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int i = lane + KVF_WAVE * j, e = 2 * i;
+      if (e >= a.d) continue;
+      float y0 = e < dk ? u[j] * r * w[e] : 0.f;
+      float y1 = e + 1 < dk ? v[j] * r * w[e + 1] : 0.f;
+      if (e < a.rot && pos_ok && cs) {
+        const float c = cs[i], sv = sn[i];
+        const float t0 = y0 * c - y1 * sv, t1 = y1 * c + y0 * sv;
+        y0 = t0;
+        y1 = t1;
+      }
+      Elem<T>::store(dst + e, y0);
+      if (e + 1 < a.d) Elem<T>::store(dst + e + 1, y1);
+    }
+  }
+  if (page < 0) return;
+  for (int t = threadIdx.x; t < a.KV * a.d; t += blockDim.x) {
+    const int hh = t / a.d, i = t - hh * a.d;
+    v_pages[((static_cast<size_t>(page) * a.KV + hh) * a.d + i) * a.block_size + off] =
+        row[(a.H + a.KV + hh) * a.d + i];
+  }
+}
+
+template <typename T>
+static int qknorm_rope_launch(void* qkv, const int* positions, const int* seq_of_token, const float* cos_t,
+                              const float* sin_t, const int* block_table, void* k_pages, void* v_pages,
+                              const float* qw, const float* kw, int dk, float eps, int n, RopeArgs a,
+                              hipStream_t s) {
+  if (n <= 0) return 0;
+  if (a.d > 4 * KVF_WAVE || dk > a.d || dk <= 0 || a.rot > dk || a.rot % 2 || !qw || (a.write_kv && !kw))
+    return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<T>, dim3(n), dim3(256), 0, s, static_cast<T*>(qkv), positions,
+                     seq_of_token, cos_t, sin_t, block_table, static_cast<T*>(k_pages),
+                     static_cast<T*>(v_pages), qw, kw, dk, eps, a);
+  return kvf_last_error();
+}
+#define QKNORM_ARGS_DECL                                                                         \
+  void *qkv, const int *positions, const int *seq_of_token, const float *cos_t,                 \
+      const float *sin_t, const int *block_table, void *k_pages, void *v_pages, const float *qw, \
+      const float *kw, int dk, float eps, int n, int H, int KV, int d, int rot, int table_len,   \
+      int block_size, int table_stride, int num_blocks, int write_kv, int n_seqs, int row_len,   \
+      hipStream_t s
+KVF_EXPORT int kvf_qknorm_rope_kvwrite_f32(QKNORM_ARGS_DECL) {
+  return qknorm_rope_launch<float>(qkv, positions, seq_of_token, cos_t, sin_t, block_table, k_pages,
+                                   v_pages, qw, kw, dk, eps, n, ROPE_ARGS_PACK, s);
+}
+KVF_EXPORT int kvf_qknorm_rope_kvwrite_bf16(QKNORM_ARGS_DECL) {
+  return qknorm_rope_launch<bf16_t>(qkv, positions, seq_of_token, cos_t, sin_t, block_table, k_pages,
+                                    v_pages, qw, kw, dk, eps, n, ROPE_ARGS_PACK, s);
+}
+
+// ----------------------------------------------------------------------------- soft cap
+// x = cap * tanh(x / cap) over fp32 values (logits), in place.
+__global__ void softcap_kernel(float* __restrict__ x, long total, float cap) {
+  const long i = static_cast<long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i < total) x[i] = cap * tanhf(x[i] / cap);
+}
+KVF_EXPORT int kvf_softcap(float* x, long total, float cap, hipStream_t s) {
+  if (total <= 0) return 0;
+  if (!(cap > 0.f)) return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(softcap_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, s, x,
+                     total, cap);
+  return kvf_last_error();
 }
 
 // ----------------------------------------------------------------------------- learned positions

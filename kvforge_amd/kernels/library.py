@@ -44,6 +44,8 @@ MODULES: dict[str, list[str]] = {
     "attn_mfma": ["attn_mfma.hip"],
     "sampling": ["sampling.hip"],
     "gemm_library": ["gemm_library.hip"],
+    "mlstm": ["mlstm.hip"],
+    "moe": ["moe.hip"],
 }
 
 

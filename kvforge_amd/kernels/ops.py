@@ -100,16 +100,25 @@ def _fn(module: str, name: str, argtypes: list):
 
 
 # ------------------------------------------------------------------------------ embedding
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
-    """``out[n] = table[ids[n]]`` widened to fp32 (the residual stream)."""
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+    """``out[n] = table[ids[n]] * scale``, widened to fp32 first (the residual stream)."""
     n = ids.shape[0]
     _check(ids, "ids", I32, (n,))
     _check(table, "table", None, (None, None))
     vocab, h = table.shape
     _check(out, "out", F32, (n, h))
     f = _fn("elementwise", f"kvf_embed_{_suffix(table.dtype)}",
-            [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p])
-    _ok(f(ids.data_ptr(), table.data_ptr(), out.data_ptr(), n, h, vocab, _stream()), "embed")
+            [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_void_p])
+    _ok(f(ids.data_ptr(), table.data_ptr(), out.data_ptr(), n, h, vocab, float(scale), _stream()), "embed")
+
+
+def softcap(x: torch.Tensor, cap: float) -> None:
+    """``x = cap * tanh(x / cap)`` in place over fp32 values (logits)."""
+    _check(x, "x", F32)
+    if not cap > 0.0:
+        raise KernelError(f"softcap: the cap must be positive, got {cap}")
+    f = _fn("elementwise", "kvf_softcap", [c_void_p, c_long, c_float, c_void_p])
+    _ok(f(x.data_ptr(), x.numel(), float(cap), _stream()), "softcap")
 
 
 # ------------------------------------------------------------------------------ RMS norm
@@ -402,6 +411,44 @@ def rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch
           n, H, KV, d, rot, table_len, bs, stride, nb, 1 if write_kv else 0, n_seqs,
           qkv.shape[1], _stream()),
         "rope_kvwrite")
+
+
+def qknorm_rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, seq_of_token: torch.Tensor,
+                        cos: torch.Tensor | None, sin: torch.Tensor | None, block_table: torch.Tensor,
+                        k_pages: torch.Tensor, v_pages: torch.Tensor, num_heads: int,
+                        num_kv_heads: int, head_dim: int, q_weight: torch.Tensor,
+                        k_weight: torch.Tensor, norm_dim: int, eps: float, write_kv: bool = True) -> None:
+    """``rope_kvwrite`` with a norm per head in front of the rotation: every q and k head is
+    divided by the root mean square of its first ``norm_dim`` elements (``eps`` inside the root)
+    and multiplied by ``q_weight`` / ``k_weight`` (fp32 ``[norm_dim]``, shared by the heads), in
+    fp32 from the projected row; elements ``norm_dim..head_dim-1`` (padding) stay zero."""
+    n = qkv.shape[0]
+    H, KV, d = num_heads, num_kv_heads, head_dim
+    _check(qkv, "qkv", None, (n, None))
+    if qkv.shape[1] < (H + 2 * KV) * d:
+        raise KernelError(f"qknorm_rope_kvwrite: rows of {qkv.shape[1]} elements do not hold q, k and v")
+    if not 0 < norm_dim <= d <= 256:
+        raise KernelError(f"qknorm_rope_kvwrite: norm over {norm_dim} of {d} elements (at most 256)")
+    _check(positions, "positions", I32, (None,))
+    _check(seq_of_token, "seq_of_token", I32, (None,))
+    if positions.shape[0] < n or seq_of_token.shape[0] < n:
+        raise KernelError("qknorm_rope_kvwrite: positions / seq_of_token shorter than the batch")
+    cos_p, sin_p, rot, table_len = _rotary_tables(cos, sin, d, "qknorm_rope_kvwrite")
+    if rot > norm_dim:
+        raise KernelError(f"qknorm_rope_kvwrite: rotary width {rot} beyond the head's {norm_dim} elements")
+    _check(q_weight, "q_weight", F32, (norm_dim,))
+    _check(k_weight, "k_weight", F32, (norm_dim,))
+    _check(block_table, "block_table", I32, (None, None))
+    n_seqs, stride = block_table.shape
+    _check(k_pages, "k_pages", qkv.dtype, (None, KV, None, d))
+    nb, _, bs, _ = k_pages.shape
+    _check(v_pages, "v_pages", qkv.dtype, (nb, KV, d, bs))
+    f = _fn("elementwise", f"kvf_qknorm_rope_kvwrite_{_suffix(qkv.dtype)}",
+            [c_void_p] * 10 + [c_int, c_float] + [c_int] * 12 + [c_void_p])
+    _ok(f(qkv.data_ptr(), positions.data_ptr(), seq_of_token.data_ptr(), cos_p, sin_p,
+          block_table.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), q_weight.data_ptr(),
+          k_weight.data_ptr(), int(norm_dim), float(eps), n, H, KV, d, rot, table_len, bs, stride, nb,
+          1 if write_kv else 0, n_seqs, qkv.shape[1], _stream()), "qknorm_rope_kvwrite")
 
 
 # ------------------------------------------------------------------------------ matrix products
@@ -880,6 +927,16 @@ def _slopes_ptr(slopes, H: int, like: torch.Tensor):
     return slopes.data_ptr()
 
 
+def _sinks_ptr(sinks, H: int, like: torch.Tensor):
+    """Pointer to the per-head sink scores (fp32 ``[H]``), or ``None`` for a softmax without."""
+    if sinks is None:
+        return None
+    _check(sinks, "sinks", F32, (H,))
+    if sinks.device != like.device:
+        raise KernelError("attention: sinks live on another device than q")
+    return sinks.data_ptr()
+
+
 def _keep_first(window: int, keep_first: int) -> int:
     """Keys kept visible behind a window; without a window every key is visible anyway."""
     keep = int(keep_first)
@@ -934,7 +991,8 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  work: torch.Tensor, out: torch.Tensor, num_heads: int, num_kv_heads: int,
                  head_dim: int, scale: float, window: int = 0,
                  slopes: torch.Tensor | None = None, rows_per_item: int | None = None,
-                 keep_first: int = 0, gate: torch.Tensor | None = None) -> None:
+                 keep_first: int = 0, gate: torch.Tensor | None = None,
+                 sinks: torch.Tensor | None = None) -> None:
     """Causal attention of query runs over the paged cache.  ``work``: ``[num_work, 3]`` rows
     (sequence row, item, item or -1) where a sequence has ``query_len * H/KV`` rows per kv head,
     an item covers ``rows_per_item`` of them (what ``prefill_rows_per_item`` gave when the rows
@@ -945,23 +1003,26 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     ``keep_first``: with a window, the first so many keys of a sequence stay visible behind it.
     ``gate`` (``[tokens, H*d]``, dense rows, type of ``q``): an output gate; what is stored is the
     attention output times ``sigmoid(gate)``, element by element, in the matrix-core kernels'
-    store (the 32-bit kernels take no gate: their caller runs ``sigmoid_gate`` behind them)."""
+    store (the 32-bit kernels take no gate: their caller runs ``sigmoid_gate`` behind them).
+    ``sinks``: fp32 ``[H]``; the softmax's denominator of head ``h`` then holds one more term
+    ``exp(sinks[h])``, a key without a value whose score is not scaled."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     _check(work, "work", I32, (None, 3))
     keep = _keep_first(window, keep_first)
     gp, gs = _gate_args(gate, q, H * d)
     sl = _slopes_ptr(slopes, H, q)
+    sk = _sinks_ptr(sinks, H, q)
     nb, _, bs, _ = k_pages.shape
     if rows_per_item is None:
         rows_per_item = prefill_rows_per_item(q.dtype, d, bs)
     if attention_on_matrix_cores(q.dtype, bs):
         f = _fn("attn_mfma", "kvf_attn_mfma_prefill",
-                [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 11 + [c_float, c_void_p, c_void_p, c_int, c_void_p])
+                [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 11 + [c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p])
         _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
               cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(), work.shape[0], int(rows_per_item), out.data_ptr(),
               H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0), int(window), keep,
-              n_seqs, float(scale), sl, gp, gs, _stream()), "attn_mfma_prefill")
+              n_seqs, float(scale), sl, gp, gs, sk, _stream()), "attn_mfma_prefill")
         return
     if gate is not None:
         raise KernelError("attn_prefill: the 32-bit kernel takes no gate; gate its rows afterwards")
@@ -972,11 +1033,11 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
         raise KernelError("attn_prefill: rows of q and out must start on 16 bytes")
     f = _fn("attn_generic", "kvf_attn_generic",
             [c_int] + [c_void_p] * 7 + [c_int] + [c_void_p] + [c_int] * 11
-            + [c_float, c_void_p, c_void_p])
+            + [c_float, c_void_p, c_void_p, c_void_p])
     _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
           block_table.data_ptr(), cu_q.data_ptr(), ctx_lens.data_ptr(), work.data_ptr(),
           work.shape[0], out.data_ptr(), H, KV, d, bs, nb, block_table.shape[1], q.stride(0),
-          out.stride(0), int(window), keep, n_seqs, float(scale), sl, _stream()), "attn_generic")
+          out.stride(0), int(window), keep, n_seqs, float(scale), sl, sk, _stream()), "attn_generic")
 
 
 def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
@@ -985,7 +1046,8 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                 num_kv_heads: int, head_dim: int, scale: float, window: int = 0, splits: int = 1,
                 workspace: tuple[torch.Tensor, torch.Tensor] | None = None,
                 token_is_seq: bool = False, slopes: torch.Tensor | None = None,
-                keep_first: int = 0, gate: torch.Tensor | None = None) -> None:
+                keep_first: int = 0, gate: torch.Tensor | None = None,
+                sinks: torch.Tensor | None = None) -> None:
     """Attention of one-token queries: sequence rows ``seq_ids[:num_seqs]`` (or ``0..num_seqs-1``)
     each attend from their token ``cu_q[seq]`` over ``ctx_lens[seq]`` cached keys.  The key
     range may be cut into ``splits`` runs; ``workspace`` then holds fp32 partial accumulators
@@ -993,10 +1055,12 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     ``token_is_seq``: the caller vouches that ``cu_q[i] == i`` for every sequence (a batch of
     single tokens), which spares the matrix-core kernel a dependent load.  ``slopes``: as in
     ``attn_prefill``; ``keep_first`` and ``gate`` likewise (the matrix-core kernels only: the
-    32-bit path is given no gate, its caller gates the rows afterwards)."""
+    32-bit path is given no gate, its caller gates the rows afterwards); ``sinks`` likewise (all
+    kernels; with cuts the term joins the sum where the cuts are merged)."""
     H, KV, d = num_heads, num_kv_heads, head_dim
     n_seqs = _attn_common(q, k_pages, v_pages, block_table, cu_q, ctx_lens, out, H, KV, d)
     sl = _slopes_ptr(slopes, H, q)
+    sk = _sinks_ptr(sinks, H, q)
     keep = _keep_first(window, keep_first)
     gp, gs = _gate_args(gate, q, H * d)
     if token_is_seq and seq_ids is not None:
@@ -1023,23 +1087,145 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
         if gate is not None:
             raise KernelError("attn_decode: the 32-bit kernel takes no gate; gate its rows afterwards")
         f = _fn("attn_generic", "kvf_attn_generic_decode",
-                [c_int] + [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p])
+                [c_int] + [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p, c_void_p])
         _ok(f(_tcode(q.dtype), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
               block_table.data_ptr(), seq_ids.data_ptr() if seq_ids is not None else None,
               None if token_is_seq else cu_q.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(),
               pa.data_ptr() if pa is not None else None, pm.data_ptr() if pm is not None else None,
               num_seqs, H, KV, d, bs, nb, block_table.shape[1], q.stride(0), out.stride(0),
-              int(window), keep, n_seqs, int(splits), float(scale), sl, _stream()), "attn_generic_decode")
+              int(window), keep, n_seqs, int(splits), float(scale), sl, sk, _stream()), "attn_generic_decode")
         return
     f = _fn("attn_mfma", "kvf_attn_mfma_decode",
-            [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p, c_int, c_void_p])
+            [c_void_p] * 10 + [c_int] * 13 + [c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p])
     _ok(f(q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(),
           seq_ids.data_ptr() if seq_ids is not None else None,
           None if token_is_seq else cu_q.data_ptr(),
           ctx_lens.data_ptr(), out.data_ptr(), pa.data_ptr() if pa is not None else None,
           pm.data_ptr() if pm is not None else None, num_seqs, H, KV, d, bs, nb,
           block_table.shape[1], q.stride(0), out.stride(0), int(window), keep, n_seqs, int(splits),
-          float(scale), sl, gp, gs, _stream()), "attn_mfma_decode")
+          float(scale), sl, gp, gs, sk, _stream()), "attn_mfma_decode")
+
+
+# ------------------------------------------------------------------------------ matrix-memory recurrence
+def mlstm_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
+    """fp32 numbers of one request's state: per head the matrix ``[key_dim, value_dim]``, the
+    normaliser ``[key_dim]`` and the running maximum."""
+    return heads * (key_dim * value_dim + key_dim + 1)
+
+
+def mlstm_scan(rows: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor, cu_q: torch.Tensor,
+               positions: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor,
+               num_seqs: int, heads: int, key_dim: int, value_dim: int, q_off: int, k_off: int,
+               v_off: int, cap: float, q_scale: float) -> None:
+    """The matrix-memory recurrence over every sequence's tokens of this step, from and into the
+    sequences' state slots.  ``rows [N, >= ...]``: projected rows holding q (``heads * key_dim``
+    elements from column ``q_off``), k (from ``k_off``) and v (``heads * value_dim`` from
+    ``v_off``); ``gates [N, 2 heads]`` fp32: input-gate then forget-gate pre-activations, to
+    which ``gate_bias [2 heads]`` is added before the cap ``cap * tanh(z / cap)``; the forget
+    gate's log is ``logsigmoid`` of its capped value.  ``state [slots, mlstm_state_floats]``
+    fp32; a sequence whose first token of the step sits at position 0 starts from zeros whatever
+    its slot holds; a negative slot skips the sequence.  ``out [N, heads * value_dim]`` fp32: the
+    heads' outputs ``S^T q / (max(|n . q|, exp(-m)) + 1e-6)`` with ``q`` times ``q_scale``."""
+    n = rows.shape[0]
+    H, dk, dv = int(heads), int(key_dim), int(value_dim)
+    _check(rows, "rows", None, (n, None), contiguous=False)
+    if rows.stride(1) != 1:
+        raise KernelError("mlstm_scan: rows must be dense")
+    for off, size, name in ((q_off, H * dk, "q"), (k_off, H * dk, "k"), (v_off, H * dv, "v")):
+        if off < 0 or off + size > rows.shape[1]:
+            raise KernelError(f"mlstm_scan: {name} at columns {off}..{off + size} lies outside rows of {rows.shape[1]}")
+    if not 0 < dk <= 256:
+        raise KernelError(f"mlstm_scan: key sizes up to 256, got {dk}")
+    _check(gates, "gates", F32, (n, 2 * H))
+    _check(gate_bias, "gate_bias", F32, (2 * H,))
+    _check(cu_q, "cu_q", I32, (None,))
+    _check(positions, "positions", I32, (None,))
+    _check(slot_ids, "slot_ids", I32, (None,))
+    if cu_q.shape[0] < num_seqs + 1 or slot_ids.shape[0] < num_seqs or positions.shape[0] < n:
+        raise KernelError("mlstm_scan: cu_q / slot_ids / positions shorter than the batch")
+    _check(state, "state", F32, (None, mlstm_state_floats(H, dk, dv)))
+    _check(out, "out", F32, (n, H * dv))
+    f = _fn("mlstm", "kvf_mlstm_scan", [c_int] + [c_void_p] * 8 + [c_int] * 9 + [c_float, c_float, c_void_p])
+    _ok(f(_tcode(rows.dtype), rows.data_ptr(), gates.data_ptr(), gate_bias.data_ptr(), cu_q.data_ptr(),
+          positions.data_ptr(), slot_ids.data_ptr(), state.data_ptr(), out.data_ptr(), int(num_seqs),
+          H, dk, dv, rows.stride(0) if n > 1 else rows.shape[1], int(q_off), int(k_off), int(v_off),
+          state.shape[0], float(cap), float(q_scale), _stream()), "mlstm_scan")
+
+
+def mlstm_out(heads_raw: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float,
+              out: torch.Tensor, heads: int, value_dim: int) -> None:
+    """``out[n, h, :] = o / rms(o) * weight[h, :] * sigmoid(gate[n, h, :])`` for the raw heads
+    ``o = heads_raw[n, h, :]`` (fp32): the root mean square is taken per head over its
+    ``value_dim`` elements, ``eps`` inside the root.  ``gate``: dense rows of ``out``'s type (a
+    view of wider rows is fine)."""
+    n = heads_raw.shape[0]
+    H, dv = int(heads), int(value_dim)
+    _check(heads_raw, "heads_raw", F32, (n, H * dv))
+    _check(weight, "weight", F32, (H * dv,))
+    _check(out, "out", None, (n, H * dv))
+    _check(gate, "gate", out.dtype, (n, H * dv), contiguous=False)
+    if gate.stride(1) != 1:
+        raise KernelError("mlstm_out: gate rows must be dense")
+    f = _fn("mlstm", "kvf_mlstm_out", [c_int, c_void_p, c_void_p, c_int, c_void_p, c_float, c_void_p] + [c_int] * 3 + [c_void_p])
+    _ok(f(_tcode(out.dtype), heads_raw.data_ptr(), gate.data_ptr(), gate.stride(0) if n > 1 else H * dv,
+          weight.data_ptr(), float(eps), out.data_ptr(), n, H, dv, _stream()), "mlstm_out")
+
+
+# ------------------------------------------------------------------------------ routed experts
+MOE_MAX_ROUTER_OUTPUTS = 512
+MOE_MAX_TOP = 16
+
+
+def moe_topk(logits: torch.Tensor, correction: torch.Tensor, chosen: torch.Tensor,
+             weights: torch.Tensor) -> None:
+    """The router's choice per token from its fp32 ``logits [N, R]``: ``s = softmax(logits)``, the
+    ``top`` outputs with the largest ``s + correction`` (the lowest index among equals) go to
+    ``chosen [N, top]`` (int32) and their ``s``, divided by the sum of the chosen ``s`` (+ 1e-20),
+    to ``weights [N, top]`` (fp32)."""
+    n, R = logits.shape
+    _check(logits, "logits", F32, (n, R), contiguous=False)
+    if logits.stride(1) != 1:
+        raise KernelError("moe_topk: logits rows must be dense")
+    _check(correction, "correction", F32, (R,))
+    top = chosen.shape[1]
+    _check(chosen, "chosen", I32, (n, top))
+    _check(weights, "weights", F32, (n, top))
+    if R > MOE_MAX_ROUTER_OUTPUTS or not 0 < top <= min(MOE_MAX_TOP, R):
+        raise KernelError(f"moe_topk: up to {MOE_MAX_ROUTER_OUTPUTS} router outputs and {MOE_MAX_TOP} choices, got {R} / {top}")
+    f = _fn("moe", "kvf_moe_topk", [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p])
+    _ok(f(logits.data_ptr(), logits.stride(0) if n > 1 else R, correction.data_ptr(), chosen.data_ptr(),
+          weights.data_ptr(), n, R, top, _stream()), "moe_topk")
+
+
+def moe_dense_act(gate_up: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor, out: torch.Tensor,
+                  experts: int, ff: int) -> None:
+    """``gate_up [N, 2 experts ff]`` holds every expert's (gate, up) pairs as neighbouring columns;
+    ``out[n, e ff + j] = weight(n, e) * silu(gate) * up`` where token ``n`` chose expert ``e`` and an
+    exact zero elsewhere."""
+    n = gate_up.shape[0]
+    E, top = int(experts), chosen.shape[1]
+    _check(gate_up, "gate_up", None, (n, 2 * E * ff))
+    _check(out, "out", gate_up.dtype, (n, E * ff))
+    _check(chosen, "chosen", I32, (n, top))
+    _check(weights, "weights", F32, (n, top))
+    f = _fn("moe", "kvf_moe_dense_act", [c_int] + [c_void_p] * 4 + [c_int] * 4 + [c_void_p])
+    _ok(f(_tcode(gate_up.dtype), gate_up.data_ptr(), chosen.data_ptr(), weights.data_ptr(), out.data_ptr(),
+          n, E, int(ff), top, _stream()), "moe_dense_act")
+
+
+def moe_identity(x: torch.Tensor, h: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor,
+                 first: int) -> None:
+    """``x[n] += w * h[n]`` with ``w`` the sum of the weights of token ``n``'s choices that are
+    ``>= first`` (router outputs that pass the input on); ``x`` is the fp32 stream."""
+    n, width = x.shape
+    _check(x, "x", F32, (n, width))
+    _check(h, "h", None, (n, width))
+    top = chosen.shape[1]
+    _check(chosen, "chosen", I32, (n, top))
+    _check(weights, "weights", F32, (n, top))
+    f = _fn("moe", "kvf_moe_identity", [c_int] + [c_void_p] * 4 + [c_int] * 4 + [c_void_p])
+    _ok(f(_tcode(h.dtype), x.data_ptr(), h.data_ptr(), chosen.data_ptr(), weights.data_ptr(), n, width,
+          top, int(first), _stream()), "moe_identity")
 
 
 # ------------------------------------------------------------------------------ sampling

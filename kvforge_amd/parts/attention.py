@@ -90,7 +90,14 @@ class PagedAttention(Mixer):
     their product.
     ``own_kv``: ``False`` for a mixer without key and value projections, which reads the cache
     of another call (``LayerCall.cache_of``) with queries, mask and gate of its own.
-    ``names``: checkpoint names of the matrices under the prefix, by ``q k v o g``."""
+    ``names``: checkpoint names of the matrices under the prefix, by ``q k v o g``.
+    ``qk_norm``: ``(name of q's weight, name of k's weight, eps)`` under the prefix: every q head
+    and every k head is divided by its root mean square over ``head_dim`` and multiplied by a
+    weight vector ``[head_dim]`` that the heads share, before the rotation; in fp32, in the
+    kernel that also rotates and writes the cache.
+    ``sink``: name of a tensor ``[num_heads]`` under the prefix: the softmax's denominator of
+    head ``h`` gets one more term ``exp(sink[h])`` (not scaled), which takes weight from the
+    keys and has no value."""
 
     NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
              "g": "g_proj.weight"}
@@ -102,7 +109,8 @@ class PagedAttention(Mixer):
                  rotary: RotaryPositions | None, scale: float | None = None,
                  window: int | None = None, score_slopes=None, keep_first: int = 0,
                  value_dim: int | None = None, gated: bool = False, own_kv: bool = True,
-                 names: dict[str, str] | None = None) -> None:
+                 names: dict[str, str] | None = None,
+                 qk_norm: tuple[str, str, float] | None = None, sink: str | None = None) -> None:
         if num_heads % num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         self.dk = int(head_dim)
@@ -128,6 +136,10 @@ class PagedAttention(Mixer):
         if self.score_slopes is not None and len(self.score_slopes) != self.H:
             raise ValueError(f"score_slopes needs one number per q head ({self.H}), got {len(self.score_slopes)}")
         self.slopes: torch.Tensor | None = None
+        self.qk_norm, self.sink = qk_norm, sink
+        if qk_norm is not None and not own_kv:
+            raise ValueError("a norm of q and k goes with key and value projections of the mixer's own")
+        self.q_norm_w = self.k_norm_w = self.sinks = None
         self.cache_spec = CacheSpec(attention_pages(self.KV, self.d), self.window, self.keep_first)
         self.w_qkv: torch.Tensor | None = None
         self.w_o: torch.Tensor | None = None
@@ -141,6 +153,11 @@ class PagedAttention(Mixer):
                   "g": (H * self.dv, h)}
         out = {self._name(self.names[n]): WeightSpec(shapes[n]) for n in self._matrices()}
         out[self._name(self.names["o"])] = WeightSpec((h, H * self.dv))
+        if self.qk_norm is not None:
+            out[self._name(self.qk_norm[0])] = WeightSpec((self.dk,), init="norm", std=0.1)
+            out[self._name(self.qk_norm[1])] = WeightSpec((self.dk,), init="norm", std=0.1)
+        if self.sink is not None:
+            out[self._name(self.sink)] = WeightSpec((H,), std=1.0)
         return out
 
     def _padded_heads(self, w: torch.Tensor, heads: int, size: int, perm=None) -> torch.Tensor:
@@ -178,6 +195,11 @@ class PagedAttention(Mixer):
             w_o = w_o.reshape(self.hidden, self.H * self.d).contiguous()
         self.w_o = w_o
         self.norm_eps = None
+        if self.qk_norm is not None:
+            self.q_norm_w = tensors[self._name(self.qk_norm[0])].float().contiguous()
+            self.k_norm_w = tensors[self._name(self.qk_norm[1])].float().contiguous()
+        if self.sink is not None:
+            self.sinks = tensors[self._name(self.sink)].float().contiguous()
         if self.score_slopes is not None:
             self.slopes = torch.tensor(self.score_slopes, dtype=torch.float32, device=self.w_o.device)
 
@@ -186,6 +208,8 @@ class PagedAttention(Mixer):
         elements i and i + rot/2; elements beyond the rotary width stay."""
         rot = self.rotary.rot_dim if self.rotary is not None else 0
         perm = torch.arange(self.dk)
+        if rot and getattr(self.rotary, "interleaved", False):
+            return perm      # the checkpoint's pairs are neighbours already
         for i in range(rot // 2):
             perm[2 * i], perm[2 * i + 1] = i, i + rot // 2
         return perm
@@ -203,8 +227,9 @@ class PagedAttention(Mixer):
         return type(self).after_projection is not PagedAttention.after_projection
 
     def _plain(self) -> bool:
-        """Whether the product holds q, k and v and nothing else."""
-        return self.own_kv and not self.gated
+        """Whether the product holds q, k and v and nothing else, and nothing but the rotation
+        lies between it and the cache."""
+        return self.own_kv and not self.gated and self.qk_norm is None
 
     def absorb_norm(self, norm) -> bool:
         if self._hooked() or not self._plain():
@@ -223,10 +248,13 @@ class PagedAttention(Mixer):
 
     def num_bytes(self) -> int:
         return sum(t.numel() * t.element_size()
-                   for t in map(ops.plain_of, (self.w_qkv, self.w_o)) if t is not None)
+                   for t in (*map(ops.plain_of, (self.w_qkv, self.w_o)), *self._small()) if t is not None)
+
+    def _small(self) -> list[torch.Tensor]:
+        return [t for t in (self.q_norm_w, self.k_norm_w, self.sinks) if t is not None]
 
     def held_tensors(self) -> list[torch.Tensor]:
-        return ops.copies_of(self.w_qkv) + ops.copies_of(self.w_o)
+        return ops.copies_of(self.w_qkv) + ops.copies_of(self.w_o) + self._small()
 
     def seal(self) -> None:
         self.w_qkv, self.w_o = ops.streamed(ops.plain_of(self.w_qkv)), ops.streamed(ops.plain_of(self.w_o))
@@ -301,7 +329,8 @@ class PagedAttention(Mixer):
             normed = ws.buf("normed", (n, self.hidden), act)
             ops.rmsnorm(x, None, rms, normed, add=step.take_owed(residual))
             x, rms = normed, None
-        fused = (not self._hooked() and ops.bf16_kernel_takes(x, self.w_qkv, rms is not None, True)
+        fused = (not self._hooked() and self.qk_norm is None
+                 and ops.bf16_kernel_takes(x, self.w_qkv, rms is not None, True)
                  and layer.k_pages.dtype == torch.bfloat16)
         if fused and rms is not None:
             # what the layer before owes the stream rides in this projection's loads and is
@@ -326,7 +355,12 @@ class PagedAttention(Mixer):
             qkv = ws.buf("qkv", (n, self.w_qkv.shape[0]), act)
             ops.gemm(x, self.w_qkv, qkv)
             self.after_projection(qkv, step)
-            if self.own_kv or self.rotary is not None:
+            if self.qk_norm is not None:
+                ops.qknorm_rope_kvwrite(qkv, step.positions, step.seq_of_token, cos, sin, table,
+                                        layer.k_pages, layer.v_pages, H, KV, d, self.q_norm_w,
+                                        self.k_norm_w, self.dk, self.qk_norm[2],
+                                        write_kv=layer.owns_cache)
+            elif self.own_kv or self.rotary is not None:
                 ops.rope_kvwrite(qkv, step.positions, step.seq_of_token, cos, sin, table,
                                  layer.k_pages, layer.v_pages, H, KV, d,
                                  write_kv=layer.owns_cache and self.own_kv)
@@ -340,7 +374,7 @@ class PagedAttention(Mixer):
         if work is not None:
             ops.attn_prefill(qkv, layer.k_pages, layer.v_pages, table, step.cu_q, step.ctx_lens,
                              work, out, H, KV, d, self.scale, window, self.slopes, rows_per_item,
-                             keep_first=self.keep_first, gate=gate_in_kernel)
+                             keep_first=self.keep_first, gate=gate_in_kernel, sinks=self.sinks)
         if step.n_decode:
             splits = self._decode_cuts(step, ops.attention_on_matrix_cores(act, bs))
             workspace = None
@@ -351,7 +385,8 @@ class PagedAttention(Mixer):
                             step.n_decode, step.cu_q, step.ctx_lens, out, H, KV, d, self.scale,
                             window, splits, workspace,
                             token_is_seq=step.decode_seq_ids is None and work is None,
-                            slopes=self.slopes, keep_first=self.keep_first, gate=gate_in_kernel)
+                            slopes=self.slopes, keep_first=self.keep_first, gate=gate_in_kernel,
+                            sinks=self.sinks)
         if gate is not None and gate_in_kernel is None:
             ops.sigmoid_gate(out, gate)
         add_product(step, out, self.w_o, residual, owed=owed)

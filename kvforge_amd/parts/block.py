@@ -51,7 +51,8 @@ class PreNormBlock(Block):
 class ParallelBlock(Block):
     """One norm, both sublayers read its output: ``h = norm(x); x += mixer(h) + ffn(h)`` (``ffn``
     may be ``None``), then an optional part that feeds something more into the stream
-    (``after``, called as ``after.forward(residual, step, bias=...)``).
+    (``after``, called as ``after.forward(residual, step, bias=...)``).  With ``ffn_norm`` the
+    feed-forward has a norm of its own over the same ``x``: ``x += mixer(norm(x)) + ffn(ffn_norm(x))``.
 
     ``shift_name``: checkpoint name of a vector ``mu [hidden]``; the *mixer* then reads
     ``h_t + (h_{t-1} - h_t) * mu`` instead of ``h_t`` (token shift: ``h_{t-1}`` is the previous
@@ -61,8 +62,10 @@ class ParallelBlock(Block):
     shift and the state's upkeep are one kernel."""
 
     def __init__(self, norm: Norm, mixer: Mixer, ffn: FeedForward | None, hidden: int,
-                 shift_name: str | None = None, after: Part | None = None) -> None:
+                 shift_name: str | None = None, after: Part | None = None,
+                 ffn_norm: Norm | None = None) -> None:
         self.norm, self.mixer, self.ffn, self.after = norm, mixer, ffn, after
+        self.ffn_norm = ffn_norm if ffn is not None else None
         self.hidden, self.shift_name = int(hidden), shift_name
         self.mu: torch.Tensor | None = None
         if shift_name is not None:
@@ -80,7 +83,7 @@ class ParallelBlock(Block):
         return self.mixer.state_spec
 
     def parts(self) -> list[Part]:
-        return [p for p in (self.norm, self.mixer, self.ffn, self.after) if p is not None]
+        return [p for p in (self.norm, self.ffn_norm, self.mixer, self.ffn, self.after) if p is not None]
 
     def weight_specs(self) -> dict[str, WeightSpec]:
         out = super().weight_specs()
@@ -116,6 +119,10 @@ class ParallelBlock(Block):
         else:
             self.norm.forward(residual, h, add=step.take_owed(residual))
             hs = h
+        if self.ffn_norm is not None:
+            # of the same stream as the mixer's norm: taken before the mixer adds to it
+            h = step.ws.buf("parallel_normed_ffn", shape, step.act_dtype)
+            self.ffn_norm.forward(residual, h)
         self.mixer.forward(hs, step, layer, residual)
         bias = None
         if self.ffn is not None:

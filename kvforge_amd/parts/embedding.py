@@ -9,13 +9,16 @@ from kvforge_amd.parts.base import Embedding, Head, WeightSpec
 
 
 class TokenEmbedding(Embedding):
-    """``h0 = table[ids]`` into the fp32 residual stream; no scaling.  ``tensor``: the table's
-    whole checkpoint name where it is not ``<prefix>.weight``."""
+    """``h0 = table[ids] * scale`` into the fp32 residual stream (the product in fp32; ``scale``
+    1 by default).  ``tensor``: the table's whole checkpoint name where it is not
+    ``<prefix>.weight``."""
 
     replayable = True
 
-    def __init__(self, prefix: str, vocab: int, hidden: int, tensor: str | None = None) -> None:
+    def __init__(self, prefix: str, vocab: int, hidden: int, tensor: str | None = None,
+                 scale: float = 1.0) -> None:
         self.prefix, self.vocab, self.hidden = prefix, int(vocab), int(hidden)
+        self.scale = float(scale)
         self.tensor = tensor if tensor is not None else self._name("weight")
         self.table: torch.Tensor | None = None
 
@@ -32,23 +35,25 @@ class TokenEmbedding(Embedding):
         return [] if self.table is None else [self.table]
 
     def forward(self, ids: torch.Tensor, out: torch.Tensor) -> None:
-        ops.embed(ids, self.table, out)
+        ops.embed(ids, self.table, out, self.scale)
 
     def pick_table(self) -> torch.Tensor | None:
         t = self.table
-        return t if t is not None and t.dtype == torch.bfloat16 else None
+        return t if t is not None and t.dtype == torch.bfloat16 and self.scale == 1.0 else None
 
 
 class LMHead(Head):
     """``logits = x @ W^T`` in fp32 output.  ``tied_to``: the checkpoint name of the embedding
     table when the head shares it (then no tensor of its own is expected).  ``tensor``: the
-    matrix's whole checkpoint name where it is not ``<prefix>.weight``."""
+    matrix's whole checkpoint name where it is not ``<prefix>.weight``.  ``softcap``: the logits
+    become ``softcap * tanh(logits / softcap)`` (``None``: as they are)."""
 
     replayable = True
 
     def __init__(self, prefix: str, vocab: int, hidden: int, tied_to: str | None = None,
-                 tensor: str | None = None) -> None:
+                 tensor: str | None = None, softcap: float | None = None) -> None:
         self.prefix, self.vocab, self.hidden, self.tied_to = prefix, int(vocab), int(hidden), tied_to
+        self.softcap = float(softcap) if softcap else None
         self.tensor = tied_to if tied_to is not None else (tensor if tensor is not None else self._name("weight"))
         self.weight: torch.Tensor | None = None
 
@@ -59,7 +64,8 @@ class LMHead(Head):
         self.weight = tensors[self.tensor]
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
-        return {"gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())
+        return ({"gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())
+                | ({"elementwise"} if self.softcap else set()))
 
     def num_bytes(self) -> int:
         w = ops.plain_of(self.weight)
@@ -74,11 +80,15 @@ class LMHead(Head):
 
     def forward(self, x: torch.Tensor, logits: torch.Tensor) -> None:
         ops.gemm(x, self.weight, logits)
+        if self.softcap:
+            ops.softcap(logits, self.softcap)
 
     def can_pick(self, rows: int) -> bool:
-        """Whether ``pick`` takes so many rows with this weight."""
+        """Whether ``pick`` takes so many rows with this weight.  Never under a soft cap: where
+        the cap saturates, equal capped logits go to the lowest index, which the pick among the
+        raw ones would not reproduce."""
         return (isinstance(self.weight, ops.StreamedWeight) and 0 < rows <= ops.FUSED_NORM_MAX_M
-                and self.hidden % 8 == 0)
+                and self.hidden % 8 == 0 and not self.softcap)
 
     def pick(self, x: torch.Tensor, residual: torch.Tensor, step, tail) -> None:
         """The tail of a greedy decode step in one kernel (``ops.gemm_pick``): ``x`` holds the

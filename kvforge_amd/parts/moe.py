@@ -1,0 +1,124 @@
+"""Feed-forward of routed experts: every token is sent to a few of many small gated
+feed-forwards, chosen by a softmax router, plus (optionally) one that all tokens share.
+
+Router: ``s = softmax(W_r x)`` over all its outputs, in fp32.  The ``top`` outputs with the
+largest ``s + correction`` are chosen; their weights are their ``s`` divided by the sum of the
+chosen ``s`` (+ 1e-20), so the correction steers the choice and never the weights.  The router's
+last ``identity`` outputs name no expert: choosing one passes the token's input on, times the
+weight.  An expert is ``down(silu(gate x) * (up x))`` without biases; the layer's output is the
+weighted sum over the chosen experts, plus the shared expert's output.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from kvforge_amd.kernels import ops
+from kvforge_amd.parts.base import FeedForward, WeightSpec, add_product
+from kvforge_amd.parts.feedforward import GatedFeedForward
+from kvforge_amd.registry import register_feed_forward
+
+
+@register_feed_forward("moe")
+class RoutedExperts(FeedForward):
+    """``names``: checkpoint names under the prefix, by ``expert`` (a format with ``{e}``),
+    ``gate up down`` (under an expert and under ``shared``), ``router correction shared``."""
+
+    NAMES = {"expert": "e{e}", "gate": "gate", "up": "up", "down": "down", "router": "router",
+             "correction": "correction", "shared": "shared"}
+
+    replayable = True
+
+    def __init__(self, prefix: str, hidden: int, ff: int, experts: int, top: int, identity: int = 0,
+                 shared_ff: int = 0, names: dict[str, str] | None = None) -> None:
+        self.prefix, self.hidden, self.ff = prefix, int(hidden), int(ff)
+        self.E, self.top, self.identity = int(experts), int(top), int(identity)
+        self.R = self.E + self.identity
+        if not 0 < self.top <= min(self.R, ops.MOE_MAX_TOP) or self.R > ops.MOE_MAX_ROUTER_OUTPUTS:
+            raise ValueError(f"router of {self.R} outputs choosing {self.top}: the kernels take up to "
+                             f"{ops.MOE_MAX_ROUTER_OUTPUTS} outputs and {ops.MOE_MAX_TOP} choices")
+        self.names = dict(self.NAMES, **(names or {}))
+        self.shared = None
+        if shared_ff:
+            self.shared = GatedFeedForward(
+                self._name(self.names["shared"]), hidden, shared_ff, activation="silu",
+                names={k: self.names[k] for k in ("gate", "up", "down")})
+        self.w_router = self.correction = self.w_gate_up = self.w_down = None
+
+    def _expert(self, e: int, which: str) -> str:
+        return self._name(f"{self.names['expert'].format(e=e)}.{self.names[which]}")
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        h, ff = self.hidden, self.ff
+        out = {self._name(self.names["router"]): WeightSpec((self.R, h)),
+               self._name(self.names["correction"]): WeightSpec((self.R,))}
+        for e in range(self.E):
+            out[self._expert(e, "gate")] = WeightSpec((ff, h))
+            out[self._expert(e, "up")] = WeightSpec((ff, h))
+            out[self._expert(e, "down")] = WeightSpec((h, ff))
+        if self.shared is not None:
+            out.update(self.shared.weight_specs())
+        return out
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        self.w_router = tensors[self._name(self.names["router"])].float().contiguous()
+        self.correction = tensors[self._name(self.names["correction"])].float().contiguous()
+        pairs, downs = [], []
+        for e in range(self.E):
+            g, u = tensors[self._expert(e, "gate")], tensors[self._expert(e, "up")]
+            d = tensors[self._expert(e, "down")]
+            if not (g.dtype == u.dtype == d.dtype):
+                g, u, d = g.float(), u.float(), d.float()
+            # an expert's gate and up rows interleaved, the experts one after the other
+            pairs.append(torch.stack([g, u], dim=1).reshape(2 * self.ff, self.hidden))
+            downs.append(d)
+        if len({p.dtype for p in pairs}) > 1:
+            pairs, downs = [p.float() for p in pairs], [d.float() for d in downs]
+        self.w_gate_up = torch.cat(pairs, dim=0).contiguous()          # [E 2 ff, hidden]
+        self.w_down = torch.cat(downs, dim=1).contiguous()             # [hidden, E ff]
+        if self.shared is not None:
+            self.shared.load(tensors)
+
+    def seal(self) -> None:
+        self.w_gate_up = ops.streamed(ops.plain_of(self.w_gate_up))
+        self.w_down = ops.streamed(ops.plain_of(self.w_down))
+        if self.shared is not None:
+            self.shared.seal()
+
+    def kernel_modules(self, dtype: torch.dtype) -> set[str]:
+        mods = {"moe", "elementwise", "gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())
+        return mods | (self.shared.kernel_modules(dtype) if self.shared is not None else set())
+
+    def num_bytes(self) -> int:
+        """What one token reads: the router, its ``top`` experts' share of the experts' matrices,
+        the shared expert."""
+        experts = sum(t.numel() * t.element_size() for t in map(ops.plain_of, (self.w_gate_up, self.w_down))
+                      if t is not None)
+        small = sum(t.numel() * t.element_size() for t in (self.w_router, self.correction) if t is not None)
+        return (small + experts * min(self.top, self.E) // max(self.E, 1)
+                + (self.shared.num_bytes() if self.shared is not None else 0))
+
+    def held_tensors(self) -> list[torch.Tensor]:
+        return (ops.copies_of(self.w_gate_up) + ops.copies_of(self.w_down)
+                + [t for t in (self.w_router, self.correction) if t is not None]
+                + (self.shared.held_tensors() if self.shared is not None else []))
+
+    def forward(self, x, step, residual) -> None:
+        """``x``: normalised activations."""
+        n = x.shape[0]
+        ws, dt = step.ws, step.act_dtype
+        step.settle()
+        logits = ws.buf("moe_logits", (n, self.R), torch.float32)
+        ops.gemm(x, self.w_router, logits)          # a 32-bit product: the router's matrix is fp32
+        chosen = ws.buf("moe_chosen", (n, self.top), torch.int32)
+        weights = ws.buf("moe_weights", (n, self.top), torch.float32)
+        ops.moe_topk(logits, self.correction, chosen, weights)
+        if self.identity:
+            ops.moe_identity(residual, x, chosen, weights, self.E)
+        gu = ws.buf("moe_gate_up", (n, 2 * self.E * self.ff), dt)
+        ops.gemm(x, self.w_gate_up, gu)
+        act = ws.buf("moe_act", (n, self.E * self.ff), dt)
+        ops.moe_dense_act(gu, chosen, weights, act, self.E, self.ff)
+        add_product(step, act, self.w_down, residual)
+        if self.shared is not None:
+            self.shared.forward(x, step, residual)

@@ -45,6 +45,26 @@ class RMSNorm(Norm):
                 and matrix.dtype == torch.bfloat16 and matrix.shape[1] == self.width)
 
 
+@register_norm("rmsnorm_one_plus")
+class OnePlusRMSNorm(RMSNorm):
+    """RMS norm whose stored weight lies around zero: ``y = x * rsqrt(mean(x^2) + eps) * (1 + w)``.
+    The checkpoint holds ``w [width]`` under ``name``; ``1 + w`` is formed once at load in fp32
+    and kept in fp32, which is what the norm kernels multiply by."""
+
+    def __init__(self, name: str, width: int, eps: float) -> None:
+        super().__init__("", width, eps)
+        self.name = name
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        return {self.name: WeightSpec((self.width,), init="normal", std=0.1)}
+
+    def load(self, tensors: dict[str, torch.Tensor]) -> None:
+        self.weight = (1.0 + tensors[self.name].float()).contiguous()
+
+    def foldable_into(self, matrix: torch.Tensor) -> bool:
+        return False
+
+
 @register_norm("rmsnorm_scalar")
 class ScalarRMSNorm(RMSNorm):
     """RMS norm whose gain is one number for all coordinates: ``y = x * rsqrt(mean(x^2) + eps) * g``.

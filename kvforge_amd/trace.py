@@ -43,7 +43,8 @@ def main(argv: list[str] | None = None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
-    ap.add_argument("--max-live", type=int, default=16, help="most requests live at a time")
+    ap.add_argument("--max-live", type=int, default=4,
+                    help="most requests live at a time (also the number of state slots)")
     args = ap.parse_args(argv)
     if args.block_size < 1 or args.max_live < 1 or args.max_tokens < 1:
         ap.error("--block-size, --max-live and --max-tokens must be positive")
