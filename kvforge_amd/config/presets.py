@@ -88,6 +88,67 @@ PRESETS["fogorax-1b"] = fogorax(vocab=128256, width=2048, layers=16, heads=32, k
                                 ff=8192, window=1024, keep_first=4, side_dim=64, max_positions=131072)
 
 
+def rudorax(vocab: int, width: int, layers: list, loop: "tuple[int, int, int] | None" = None,
+            embedding_scale: float = 1.0, logit_softcap: float | None = None, eps: float = 1e-6,
+            max_positions: int | None = None) -> dict[str, Any]:
+    """A Rudorax config.json.  ``layers``: one ``(type, mixer, mlp)`` per layer.  For
+    ``"attention"`` the mixer holds ``heads kv_heads dim vdim window rot_dims scale scaling``
+    (``scaling``: ``None`` or the YaRN numbers ``factor original fast slow``) and optionally
+    ``base``; for ``"mlstm"`` it holds ``heads dim vdim gate_cap``.  ``mlp``: ``None`` or
+    ``ff experts top identity shared_ff``.  ``loop``: ``(start, stop, times)``."""
+    out = []
+    for kind, m, f in layers:
+        if kind == "attention":
+            mixer: dict[str, Any] = {
+                "dim": m["dim"], "heads": m["heads"], "kv_heads": m["kv_heads"], "mask": {"size": m["window"]},
+                "rot": {"base": float(m.get("base", 10000.0)), "dims": m["rot_dims"], "scaling": m.get("scaling")},
+                "scale": float(m["scale"]), "vdim": m["vdim"]}
+        else:
+            mixer = {"dim": m["dim"], "gate_cap": float(m["gate_cap"]), "heads": m["heads"], "vdim": m["vdim"]}
+        mlp = None
+        if f is not None:
+            mlp = {"expert": {"ff": f["ff"]}, "kind": "moe",
+                   "router": {"experts": f["experts"], "identity": f.get("identity", 0), "top": f["top"]},
+                   "shared": {"ff": f["shared_ff"]} if f.get("shared_ff") else None}
+        out.append({"mixer": mixer, "mlp": mlp, "type": kind})
+    cfg: dict[str, Any] = {
+        "architecture": "Rudorax", "embedding": {"scale": float(embedding_scale)}, "layers": out,
+        "logit_softcap": logit_softcap,
+        "loop": {"start": loop[0], "stop": loop[1], "times": loop[2]} if loop else None,
+        "norm": {"eps": eps}, "vocab": vocab, "width": width}
+    if max_positions is not None:
+        cfg["max_positions"] = max_positions
+    return cfg
+
+
+def rudorax_stack(vocab: int, width: int, pairs: int, heads: int, kv_heads: int, dim: int, window: int,
+                  lstm_heads: int, lstm_dim: int, lstm_vdim: int, ff: int, experts: int, top: int,
+                  identity: int, shared_ff: int, max_positions: int = 131072) -> dict[str, Any]:
+    """``pairs`` times an attention layer followed by a matrix-memory layer, all with routed
+    experts; the whole head rotated with frequencies stretched eightfold."""
+    att = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, window=window, rot_dims=dim,
+               scale=float(dim) ** -0.5, base=500000.0,
+               scaling={"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0})
+    rec = dict(heads=lstm_heads, dim=lstm_dim, vdim=lstm_vdim, gate_cap=15.0)
+    moe = dict(ff=ff, experts=experts, top=top, identity=identity, shared_ff=shared_ff)
+    return rudorax(vocab, width, [("attention", att, moe), ("mlstm", rec, moe)] * pairs,
+                   embedding_scale=float(width) ** 0.5, logit_softcap=30.0, max_positions=max_positions)
+
+
+PRESETS["rudorax-tiny"] = rudorax(
+    vocab=320, width=96,
+    layers=[("attention", dict(heads=4, kv_heads=2, dim=32, vdim=32, window=48, rot_dims=16, scale=32 ** -0.5,
+                               scaling={"factor": 4.0, "original": 64, "fast": 16.0, "slow": 1.0}),
+             dict(ff=48, experts=6, top=2, identity=1, shared_ff=64)),
+            ("mlstm", dict(heads=2, dim=24, vdim=48, gate_cap=10.0),
+             dict(ff=48, experts=6, top=2, identity=1, shared_ff=64))],
+    loop=(0, 2, 2), embedding_scale=96 ** 0.5, logit_softcap=25.0, max_positions=1024)
+# layers of the width of llama-1b: what this design's kernels are measured at
+PRESETS["rudorax-1b"] = rudorax_stack(vocab=128256, width=2048, pairs=8, heads=32, kv_heads=8, dim=64,
+                                      window=1024, lstm_heads=8, lstm_dim=128, lstm_vdim=256, ff=1024,
+                                      experts=32, top=4, identity=2, shared_ff=2048)
+
+
 def preset_dict(name: str) -> dict[str, Any]:
     try:
         return dict(PRESETS[name])

@@ -38,9 +38,15 @@ __global__ __launch_bounds__(ROWS > KVF_WAVE ? 2 * KVF_WAVE : KVF_WAVE) void mls
   const int seq = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * COLS;
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE, RG = blockDim.x / KVF_WAVE;
   const int slot = slot_ids[seq];
-  if (slot < 0 || slot >= a.n_slots) return;   // the same for the whole workgroup
   const int t0 = cu_q[seq], t1 = cu_q[seq + 1];
   if (t1 <= t0) return;
+  if (slot < 0 || slot >= a.n_slots) {   // the same for the whole workgroup
+    // a sequence without a slot (the padding of a captured batch): zeros, so that its rows
+    // never hold what an earlier step left there
+    if (wave == 0 && col0 + lane < a.dv)
+      for (int t = t0; t < t1; ++t) out[static_cast<size_t>(t) * a.H * a.dv + head * a.dv + col0 + lane] = 0.f;
+    return;
+  }
   const int dk = a.dk, dv = a.dv;
   float* ks = lds;                    // [TB][dk]
   float* qs = ks + TB * dk;           // [TB][dk]
