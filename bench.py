@@ -6,6 +6,7 @@
     python bench.py --phase mixed --preset llama-3b --batch 32 --steps 256
     python bench.py --phase burst --preset small [--dtype float32]
     python bench.py --phase fogorax [--dtype float32] [--steps 64] [--batch 8]
+    python bench.py --phase rudorax [--sizes w1024,w2048] [--steps 64] [--batch 8]
 
 Default run: the layer sizes of Llama 3.2 1B (16 layers, hidden 2048, 32 heads, 8 kv heads, head
 size 64, SwiGLU 8192, vocabulary 128256, llama3 rope scaling, tied embeddings), random weights
@@ -25,6 +26,9 @@ weights on the device.
 decode (at ``--batch`` over ``--prompt-len``-token prompts) and a 2,048-token prefill at a few
 layer sizes, each beside a Llama model of equal sizes whose layers all have the same sliding
 window, the engine's closest existing model.
+``--phase rudorax`` does the same for the Rudorax design (window attention and matrix-memory
+layers in turn, routed experts), beside a Llama model whose dense feed-forward is as wide as
+what a Rudorax token uses.
 Peaks are the published MI355X ones: HBM 8 TB/s; dense MFMA 2.5 PFLOP/s for bf16, 157.3 TFLOP/s
 for fp32.
 """
@@ -426,6 +430,73 @@ def fogorax_points(dtype, batch, prompt_len, steps, warmup, use_graphs=True):
     return out
 
 
+# (name, width, q heads, kv heads, head size, recurrent heads, their key size, their value size,
+#  expert width, experts, chosen, identity outputs, shared width, layers, vocabulary)
+RUDORAX_SIZES = [("w1024", 1024, 16, 4, 64, 4, 128, 256, 512, 16, 2, 2, 1024, 8, 32000),
+                 ("w2048", 2048, 32, 8, 64, 8, 128, 256, 1024, 32, 4, 2, 2048, 8, 128256),
+                 ("w4096", 4096, 32, 8, 128, 8, 256, 512, 2048, 32, 4, 2, 4096, 4, 128256)]
+RUDORAX_WINDOW = 1024
+
+
+def rudorax_points(dtype, batch, prompt_len, steps, warmup, use_graphs=True, only=None):
+    """Rudorax at a few sizes that resemble a real model's layers (attention and matrix-memory
+    layers in turn, routed experts in all), beside a Llama model of the same width, heads and
+    window whose dense feed-forward is as wide as what a Rudorax token uses (its chosen experts
+    plus the shared one); random weights drawn on the device.  Per size and model: ms per decode
+    step, its share of the HBM roofline, tokens a second of a 2,048-token prefill and its share
+    of the matrix-core peak.  A Rudorax decode step has to read: the mixers, routers and shared
+    experts once, the experts that the batch's tokens are expected to choose (a share
+    ``1 - (1 - top/experts)^batch`` of them), the window's keys and values, and every sequence's
+    recurrent state (read and written)."""
+    import torch
+    from kvforge_amd.config.presets import rudorax_stack
+
+    elem = 2 if dtype == "bfloat16" else 4
+    out = {}
+    for name, w, H, KV, d, Hm, dk, dv, ff, E, top, ident, shared, layers, vocab in RUDORAX_SIZES:
+        if only and name not in only:
+            continue
+        dense = top * ff + shared
+        llama = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "vocab_size": vocab,
+                 "hidden_size": w, "num_hidden_layers": layers, "num_attention_heads": H,
+                 "num_key_value_heads": KV, "head_dim": d, "intermediate_size": dense,
+                 "max_position_embeddings": CONTEXT_CAP, "rope_theta": 500000.0, "rope_scaling": None,
+                 "rms_norm_eps": 1e-5, "hidden_act": "silu", "tie_word_embeddings": False,
+                 "sliding_window": RUDORAX_WINDOW, "layer_types": ["sliding_attention"] * layers}
+        rud = rudorax_stack(vocab=vocab, width=w, pairs=layers // 2, heads=H, kv_heads=KV, dim=d,
+                            window=RUDORAX_WINDOW, lstm_heads=Hm, lstm_dim=dk, lstm_vdim=dv, ff=ff,
+                            experts=E, top=top, identity=ident, shared_ff=shared, max_positions=CONTEXT_CAP)
+        attn = w * d * (2 * H + 2 * KV)
+        lstm = w * (2 * Hm * dk + 3 * Hm * dv + 2 * Hm)
+        routed = 3 * w * ff
+        fixed = (layers // 2) * (attn + lstm) + layers * (3 * w * shared + w * (E + ident))
+        nums = {"llama": model_numbers(llama, layers),
+                "rudorax": {"linear_params": fixed + layers * top * routed, "head_params": vocab * w,
+                            "kv_values_per_token": 2 * (layers // 2) * KV * d, "attn_hd": H * d,
+                            "layers": layers // 2}}
+        touched = E * (1.0 - (1.0 - top / E) ** batch)
+        state_bytes = (layers // 2) * Hm * (dk * dv + dk + 1) * 4 * 2
+        for model, cfg in (("llama", llama), ("rudorax", rud)):
+            need = batch * (prompt_len + steps + warmup + early_tokens(batch, prompt_len) + 32)
+            engine = build_engine(cfg, dtype, batch, max(need, PREFILL_TOKENS + 64), use_graphs=use_graphs)
+            r = decode_run(engine, vocab, batch, prompt_len, steps, warmup)
+            ctx = min(r["mean_ctx"], RUDORAX_WINDOW)
+            s = prefill_run(engine, vocab, PREFILL_TOKENS, repeats=2)
+            if model == "llama":
+                read = decode_bytes(engine, nums[model], elem, batch, ctx)
+            else:
+                read = ((fixed + layers * touched * routed + vocab * w) * elem
+                        + batch * (ctx * nums[model]["kv_values_per_token"] * elem + state_bytes))
+            out[f"{name}_{model}"] = {
+                "decode_ms": round(r["ms_per_step"], 4), "decode_tok_s": round(r["tok_s"], 1),
+                "decode_hbm_frac": round(read / (r["seconds"] / steps) / 1e9 / HBM_PEAK_GBS, 4),
+                "prefill_tok_s": round(PREFILL_TOKENS / s, 1), "prefill_ms": round(s * 1e3, 3),
+                "prefill_frac": round(prefill_flops(nums[model], PREFILL_TOKENS) / s / MFMA_PEAK[dtype], 4)}
+            del engine
+            torch.cuda.empty_cache()
+    return out
+
+
 def model_numbers(cfg, layers_run):
     h, H, KV, d, I, V = (cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"],
                          cfg["head_dim"], cfg["intermediate_size"], cfg["vocab_size"])
@@ -454,7 +525,7 @@ def main() -> int:
     ap.add_argument("--no-graphs", action="store_true")
     ap.add_argument("--decode-run-steps", type=int, default=None,
                     help="decode steps the device takes between two looks of the host (engine default: 8)")
-    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed", "burst", "products", "fogorax"], default="all",
+    ap.add_argument("--phase", choices=["all", "decode", "prefill", "mixed", "burst", "products", "fogorax", "rudorax"], default="all",
                     help="for profiles: only the decode steps at --batch, or only the prefill; "
                          "mixed: --batch requests with prompts of 128 to 4,096 tokens, chunked "
                          "prefill beside decode steps, --steps new tokens each; burst: the "
@@ -462,7 +533,9 @@ def main() -> int:
                          "at once, 16 sequences a step), for --preset small or any other; "
                          "products: the four matrix products of a layer alone at --batch rows "
                          "(launch to launch, so short ones show the host's time); fogorax: the "
-                         "Fogorax design at a few layer sizes beside a Llama model of equal sizes")
+                         "Fogorax design at a few layer sizes beside a Llama model of equal sizes; "
+                         "rudorax: the Rudorax design likewise (--sizes names some of them)")
+    ap.add_argument("--sizes", default="", help="with --phase rudorax: the sizes to run, with commas")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this engine")
@@ -481,6 +554,19 @@ def main() -> int:
                                     for n, w, H, KV, d, ff, L, V, sd in FOGORAX_SIZES},
                           **fogorax_points(args.dtype, args.batch, args.prompt_len, steps,
                                            min(args.warmup, 8), not args.no_graphs)}))
+        return 0
+    if args.phase == "rudorax":
+        steps = min(args.steps, 64)
+        print(json.dumps({"phase": "rudorax", "dtype": args.dtype, "batch": args.batch,
+                          "prompt_len": args.prompt_len, "steps": steps, "window": RUDORAX_WINDOW,
+                          "prefill_tokens": PREFILL_TOKENS,
+                          "sizes": {r[0]: dict(zip(("width", "heads", "kv_heads", "head_dim", "lstm_heads",
+                                                    "lstm_dim", "lstm_vdim", "expert_ff", "experts", "top",
+                                                    "identity", "shared_ff", "layers", "vocab"), r[1:]))
+                                    for r in RUDORAX_SIZES},
+                          **rudorax_points(args.dtype, args.batch, args.prompt_len, steps,
+                                           min(args.warmup, 8), not args.no_graphs,
+                                           [x for x in args.sizes.split(",") if x] or None)}))
         return 0
     if args.preset == "small" and args.phase != "burst":
         print("--preset small goes with --phase burst")

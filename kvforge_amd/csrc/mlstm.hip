@@ -18,6 +18,8 @@ struct ScanArgs {
   int q_off, k_off, v_off;  // where q, k and v begin in a row (heads side by side)
   int n_seqs, n_slots;
   float cap, q_scale;
+  int gate_stride;          // numbers from one token's gate row to the next (at least 2 H)
+  int chunk_from;           // runs of at least so many tokens are the chunk kernel's, shorter ones the scan kernel's
 };
 
 __device__ __forceinline__ float capped(float z, float cap) { return cap * tanhf(z / cap); }
@@ -39,7 +41,7 @@ __global__ __launch_bounds__(ROWS > KVF_WAVE ? 2 * KVF_WAVE : KVF_WAVE) void mls
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE, RG = blockDim.x / KVF_WAVE;
   const int slot = slot_ids[seq];
   const int t0 = cu_q[seq], t1 = cu_q[seq + 1];
-  if (t1 <= t0) return;
+  if (t1 <= t0 || t1 - t0 >= a.chunk_from) return;   // long runs belong to the chunk kernel
   if (slot < 0 || slot >= a.n_slots) {   // the same for the whole workgroup
     // a sequence without a slot (the padding of a captured batch): zeros, so that its rows
     // never hold what an earlier step left there
@@ -87,7 +89,7 @@ __global__ __launch_bounds__(ROWS > KVF_WAVE ? 2 * KVF_WAVE : KVF_WAVE) void mls
                   : 0.f;
     }
     if (threadIdx.x < cnt) {
-      const float* z = zif + static_cast<size_t>(tb + threadIdx.x) * 2 * a.H;
+      const float* z = zif + static_cast<size_t>(tb + threadIdx.x) * a.gate_stride;
       gs[2 * threadIdx.x] = capped(z[head] + bias_if[head], a.cap);
       gs[2 * threadIdx.x + 1] = log_sigmoid(capped(z[a.H + head] + bias_if[a.H + head], a.cap));
     }
@@ -149,6 +151,247 @@ __global__ __launch_bounds__(ROWS > KVF_WAVE ? 2 * KVF_WAVE : KVF_WAVE) void mls
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same recurrence for long runs, a chunk of CL tokens at a time on the matrix cores, all in
+// fp32 (v_mfma_f32_16x16x4_f32: D[i][j] += sum_k A[i][k] B[k][j], k = 0..3; lane l gives
+// A[l % 16][l / 16] and B[l / 16][l % 16] and holds D[4 (l / 16) + v][l % 16], v = 0..3).
+//
+// With the state (S, n, m_c) at the chunk's start, b_t the sum of the log forget gates of the
+// chunk's tokens up to t, and m_t from the recurrence itself (one thread walks it, so that it is
+// the number the token-by-token kernel gets):
+//   D[t][s] = exp(b_t - b_s + li_s - m_t) for s <= t (0 otherwise),  g_t = exp(b_t + m_c - m_t)
+//   A = (Q K^T) * D;   O = A V + diag(g) Q S;   n_t . q_t = rowsum(A)_t + g_t q_t . n
+//   S' = g_L S + K^T diag(D[L]) V;   n' = g_L n + K^T D[L];   m_c' = m_L        (L: the last token)
+// which is the recurrence written out over the chunk.  A workgroup of four waves takes 64 columns
+// of S for one (sequence, head); Q, K (fp32, rows padded to an odd stride), the V columns, A and
+// the S columns live in LDS.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int CCOLS = 64;
+
+template <typename T, int DKP, int CL>
+__global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ qkv, const float* __restrict__ zif,
+                                                          const float* __restrict__ bias_if,
+                                                          const int* __restrict__ cu_q,
+                                                          const int* __restrict__ positions,
+                                                          const int* __restrict__ slot_ids,
+                                                          float* __restrict__ state, float* __restrict__ out,
+                                                          ScanArgs a) {
+  extern __shared__ float lds[];
+  constexpr int QLD = DKP + 1, ALD = CL + 1;
+  // the running sum of the log forget gates is kept in 64 bits: its differences b_t - b_s are
+  // what the weights are made of, and a sum that has passed a nearly closed gate is hundreds
+  // of times larger than the differences that matter behind it
+  double* bc = reinterpret_cast<double*>(lds);   // [CL] log forget gates, then their running sum
+  float* Qs = lds + 2 * CL;              // [CL][QLD], q times its scale
+  float* Ks = Qs + CL * QLD;             // [CL][QLD]
+  float* Vs = Ks + CL * QLD;             // [CL][CCOLS]
+  float* As = Vs + CL * CCOLS;           // [CL][ALD]
+  float* Ss = As + CL * ALD;             // [DKP][CCOLS]
+  float* ns = Ss + DKP * CCOLS;          // [DKP]
+  float* li = ns + DKP;                  // [CL] log input gates
+  float* mt = li + CL;                   // [CL] running maximum after each token
+  float* gt = mt + CL;                   // [CL] weight of the chunk's first state for token t
+  float* wl = gt + CL;                   // [CL] weight of token s in the chunk's last state
+  float* den = wl + CL;                  // [CL]
+  float* part = den + CL;                // [256 / CL][CL] shares of n . q
+  __shared__ float m_c;
+  const int seq = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * CCOLS;
+  const int tid = threadIdx.x, lane = tid % KVF_WAVE, wave = tid / KVF_WAVE;
+  const int l16 = lane % 16, lq = lane / 16;
+  const int slot = slot_ids[seq];
+  const int t0 = cu_q[seq], t1 = cu_q[seq + 1];
+  if (t1 - t0 < a.chunk_from) return;    // short runs belong to the scan kernel
+  const int dk = a.dk, dv = a.dv;
+  if (slot < 0 || slot >= a.n_slots) {
+    for (int i = tid; i < (t1 - t0) * CCOLS; i += blockDim.x) {
+      const int t = i / CCOLS, c = col0 + i % CCOLS;
+      if (c < dv) out[static_cast<size_t>(t0 + t) * a.H * dv + head * dv + c] = 0.f;
+    }
+    return;
+  }
+  const bool fresh = positions[t0] == 0;
+  float* st = state + (static_cast<size_t>(slot) * a.H + head) * (static_cast<size_t>(dk) * dv + dk + 1);
+  for (int i = tid; i < DKP * CCOLS; i += blockDim.x) {
+    const int r = i / CCOLS, c = col0 + i % CCOLS;
+    Ss[i] = (!fresh && r < dk && c < dv) ? st[static_cast<size_t>(r) * dv + c] : 0.f;
+  }
+  for (int r = tid; r < DKP; r += blockDim.x) ns[r] = (!fresh && r < dk) ? st[static_cast<size_t>(dk) * dv + r] : 0.f;
+  if (tid == 0) m_c = fresh ? 0.f : st[static_cast<size_t>(dk) * dv + dk];
+
+  for (int tb = t0; tb < t1; tb += CL) {
+    const int cnt = min(CL, t1 - tb);
+    __syncthreads();   // the chunk before is done with everything
+    for (int i = tid; i < CL * DKP; i += blockDim.x) {
+      const int t = i / DKP, e = i - t * DKP;
+      float qv = 0.f, kv = 0.f;
+      if (t < cnt && e < dk) {
+        const T* row = qkv + static_cast<size_t>(tb + t) * a.row_len;
+        qv = Elem<T>::load(row + a.q_off + head * dk + e) * a.q_scale;
+        kv = Elem<T>::load(row + a.k_off + head * dk + e);
+      }
+      Qs[t * QLD + e] = qv;
+      Ks[t * QLD + e] = kv;
+    }
+    for (int i = tid; i < CL * CCOLS; i += blockDim.x) {
+      const int t = i / CCOLS, c = col0 + i % CCOLS;
+      Vs[i] = (t < cnt && c < dv)
+                  ? Elem<T>::load(qkv + static_cast<size_t>(tb + t) * a.row_len + a.v_off + head * dv + c)
+                  : 0.f;
+    }
+    if (tid < CL) {
+      float i_gate = 0.f, f_gate = 0.f;
+      if (tid < cnt) {
+        const float* z = zif + static_cast<size_t>(tb + tid) * a.gate_stride;
+        i_gate = capped(z[head] + bias_if[head], a.cap);
+        f_gate = log_sigmoid(capped(z[a.H + head] + bias_if[a.H + head], a.cap));
+      }
+      li[tid] = i_gate;
+      bc[tid] = static_cast<double>(f_gate);
+    }
+    __syncthreads();
+    if (tid == 0) {   // the recurrence of the maximum, token by token, and the gates' running sum
+      float m = m_c;
+      double b = 0.0;
+      for (int t = 0; t < cnt; ++t) {
+        const float f = static_cast<float>(bc[t]);
+        m = fmaxf(f + m, li[t]);
+        b += static_cast<double>(f);
+        bc[t] = b;
+        mt[t] = m;
+      }
+    }
+    __syncthreads();
+    const int last = cnt - 1;
+    if (tid < CL) {
+      gt[tid] = tid < cnt ? expf(static_cast<float>(bc[tid] + static_cast<double>(m_c) - static_cast<double>(mt[tid]))) : 0.f;
+      wl[tid] = tid < cnt ? expf(static_cast<float>(bc[last] - bc[tid]) + li[tid] - mt[last]) : 0.f;
+    }
+    // ---- A = (Q K^T) * D, tile by tile; tiles above the diagonal are zero
+    constexpr int RT = CL / 16;
+    for (int tile = wave; tile < RT * RT; tile += 4) {
+      const int rt = tile / RT, ct = tile - rt * RT;
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (ct <= rt) {
+        const float* qa = Qs + (16 * rt + l16) * QLD + lq;
+        const float* kb = Ks + (16 * ct + l16) * QLD + lq;
+#pragma unroll 8
+        for (int k0 = 0; k0 < DKP; k0 += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[k0], kb[k0], acc, 0, 0, 0);
+      }
+      const int s = 16 * ct + l16;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int t = 16 * rt + 4 * lq + v;
+        const bool vis = s <= t && t < cnt;
+        As[t * ALD + s] = vis ? acc[v] * expf(static_cast<float>(bc[t] - bc[s]) + li[s] - mt[t]) : 0.f;
+      }
+    }
+    __syncthreads();
+    // ---- n . q per token: rowsum(A) + g_t q_t . n, in four shares
+    {
+      const int t = tid % CL, share = tid / CL;
+      constexpr int SH = 256 / CL;
+      float sum = 0.f;
+      for (int s2 = share; s2 < CL; s2 += SH) sum += As[t * ALD + s2];
+      float dot = 0.f;
+      for (int k = share; k < DKP; k += SH) dot = fmaf(Qs[t * QLD + k], ns[k], dot);
+      part[share * CL + t] = fmaf(gt[t], dot, sum);
+    }
+    __syncthreads();
+    if (tid < CL) {
+      constexpr int SH = 256 / CL;
+      float nq = 0.f;
+      for (int sh = 0; sh < SH; ++sh) nq += part[sh * CL + tid];
+      den[tid] = fmaxf(fabsf(nq), expf(-mt[min(tid, last)])) + 1e-6f;
+    }
+    __syncthreads();
+    // ---- O = A V + diag(g) Q S, divided by the denominator, to memory
+    for (int tile = wave; tile < RT * (CCOLS / 16); tile += 4) {
+      const int rt = tile / (CCOLS / 16), ct = tile - rt * (CCOLS / 16);
+      f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+      const float* aa = As + (16 * rt + l16) * ALD + lq;
+      const float* vb = Vs + lq * CCOLS + 16 * ct + l16;
+      for (int k0 = 0; k0 < 16 * (rt + 1); k0 += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(aa[k0], vb[k0 * CCOLS], acc, 0, 0, 0);
+      const float g = gt[16 * rt + l16];
+      const float* qa = Qs + (16 * rt + l16) * QLD + lq;
+      const float* sb = Ss + lq * CCOLS + 16 * ct + l16;
+#pragma unroll 8
+      for (int k0 = 0; k0 < DKP; k0 += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[k0] * g, sb[k0 * CCOLS], acc, 0, 0, 0);
+      const int c = col0 + 16 * ct + l16;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int t = 16 * rt + 4 * lq + v;
+        if (t < cnt && c < dv) out[static_cast<size_t>(tb + t) * a.H * dv + head * dv + c] = acc[v] / den[t];
+      }
+    }
+    __syncthreads();   // every read of S and n for this chunk is done
+    // ---- S' = g_L S + K^T diag(w) V;  n' = g_L n + K^T w
+    const float g_last = gt[last];
+    for (int tile = wave; tile < (DKP / 16) * (CCOLS / 16); tile += 4) {
+      const int kt = tile / (CCOLS / 16), ct = tile - kt * (CCOLS / 16);
+      f32x4 acc;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[v] = g_last * Ss[(16 * kt + 4 * lq + v) * CCOLS + 16 * ct + l16];
+      const float* ka = Ks + lq * QLD + 16 * kt + l16;
+      const float* vb = Vs + lq * CCOLS + 16 * ct + l16;
+#pragma unroll 8
+      for (int k0 = 0; k0 < CL; k0 += 4)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[k0 * QLD], vb[k0 * CCOLS] * wl[k0 + lq], acc, 0, 0, 0);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) Ss[(16 * kt + 4 * lq + v) * CCOLS + 16 * ct + l16] = acc[v];
+    }
+    for (int k = tid; k < DKP; k += blockDim.x) {
+      float nk = g_last * ns[k];
+      for (int s2 = 0; s2 < cnt; ++s2) nk = fmaf(wl[s2], Ks[s2 * QLD + k], nk);
+      ns[k] = nk;
+    }
+    if (tid == 0) m_c = mt[last];
+  }
+  __syncthreads();
+  for (int i = tid; i < DKP * CCOLS; i += blockDim.x) {
+    const int r = i / CCOLS, c = col0 + i % CCOLS;
+    if (r < dk && c < dv) st[static_cast<size_t>(r) * dv + c] = Ss[i];
+  }
+  if (blockIdx.x == 0) {
+    for (int r = tid; r < dk; r += blockDim.x) st[static_cast<size_t>(dk) * dv + r] = ns[r];
+    if (tid == 0) st[static_cast<size_t>(dk) * dv + dk] = m_c;
+  }
+}
+
+template <int DKP, int CL> constexpr size_t chunk_lds() {
+  return sizeof(float) * (2 * CL * (DKP + 1) + CL * CCOLS + CL * (CL + 1) + DKP * CCOLS + DKP + 7 * CL + 256);
+}
+
+template <typename T, int DKP, int CL>
+int chunk_go(const void* qkv, const float* zif, const float* bias_if, const int* cu_q, const int* positions,
+             const int* slot_ids, float* state, float* out, int num_seqs, ScanArgs a, hipStream_t s) {
+  constexpr size_t lds = chunk_lds<DKP, CL>();
+  static bool allowed = false;   // more LDS than a kernel gets unasked: asked for once per kernel
+  if (!allowed) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&mlstm_chunk_kernel<T, DKP, CL>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return static_cast<int>(e);
+    allowed = true;
+  }
+  const dim3 grid((a.dv + CCOLS - 1) / CCOLS, a.H, num_seqs);
+  hipLaunchKernelGGL((mlstm_chunk_kernel<T, DKP, CL>), grid, dim3(256), lds, s, static_cast<const T*>(qkv), zif,
+                     bias_if, cu_q, positions, slot_ids, state, out, a);
+  return kvf_last_error();
+}
+
+template <typename T>
+int chunk_launch(const void* qkv, const float* zif, const float* bias_if, const int* cu_q, const int* positions,
+                 const int* slot_ids, float* state, float* out, int num_seqs, ScanArgs a, hipStream_t s) {
+  if (num_seqs <= 0) return 0;
+#define GO(DKP, CL) return chunk_go<T, DKP, CL>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, num_seqs, a, s)
+  if (a.dk <= 32) GO(32, 64);
+  if (a.dk <= 64) GO(64, 64);
+  if (a.dk <= 128) GO(128, 64);
+  GO(256, 32);
+#undef GO
+}
+
 template <typename T>
 int scan_launch(const void* qkv, const float* zif, const float* bias_if, const int* cu_q, const int* positions,
                 const int* slot_ids, float* state, float* out, int num_seqs, ScanArgs a, hipStream_t s) {
@@ -196,20 +439,31 @@ int out_launch(const float* o, const void* g, int g_stride, const float* w, floa
 }
 }  // namespace
 
-// dtype: 0 = fp32, 1 = bf16 rows.  qkv [tokens, row_len]; zif [tokens, 2 H] fp32 (input gates,
+// dtype: 0 = fp32, 1 = bf16 rows.  qkv [tokens, row_len]; zif [tokens, gate_stride >= 2 H] fp32 (input gates,
 // then forget gates, before bias and cap); bias_if [2 H]; state [n_slots, H, dk dv + dk + 1];
 // out [tokens, H dv] fp32.  Sequence s owns tokens cu_q[s] .. cu_q[s+1]-1 and slot slot_ids[s]
 // (negative: skipped); it starts from zeros when its first token's position is 0.
+// Runs of fewer than chunk_from tokens are walked token by token (`short_runs`: launch that
+// kernel), runs of at least chunk_from tokens chunk by chunk on the matrix cores (`long_runs`);
+// each kernel leaves the other's sequences alone.
 KVF_EXPORT int kvf_mlstm_scan(int dtype, const void* qkv, const float* zif, const float* bias_if,
                               const int* cu_q, const int* positions, const int* slot_ids, float* state,
                               float* out, int num_seqs, int H, int dk, int dv, int row_len, int q_off,
-                              int k_off, int v_off, int n_slots, float cap, float q_scale, hipStream_t s) {
-  if (H <= 0 || dk <= 0 || dk > 256 || dv <= 0 || !(cap > 0.f) || num_seqs > 65535 || H > 65535)
+                              int k_off, int v_off, int n_slots, int gate_stride, float cap, float q_scale, int chunk_from,
+                              int short_runs, int long_runs, hipStream_t s) {
+  if (H <= 0 || dk <= 0 || dk > 256 || dv <= 0 || !(cap > 0.f) || num_seqs > 65535 || H > 65535 || chunk_from < 1 ||
+      gate_stride < 2 * H)
     return static_cast<int>(hipErrorInvalidValue);
-  const ScanArgs a{H, dk, dv, row_len, q_off, k_off, v_off, num_seqs, n_slots, cap, q_scale};
-  if (dtype == 0) return scan_launch<float>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, num_seqs, a, s);
-  if (dtype == 1) return scan_launch<bf16_t>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, num_seqs, a, s);
-  return static_cast<int>(hipErrorInvalidValue);
+  if (dtype != 0 && dtype != 1) return static_cast<int>(hipErrorInvalidValue);
+  const ScanArgs a{H, dk, dv, row_len, q_off, k_off, v_off, num_seqs, n_slots, cap, q_scale, gate_stride, chunk_from};
+  int code = 0;
+  if (short_runs)
+    code = dtype == 0 ? scan_launch<float>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, num_seqs, a, s)
+                      : scan_launch<bf16_t>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, num_seqs, a, s);
+  if (code == 0 && long_runs)
+    code = dtype == 0 ? chunk_launch<float>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, num_seqs, a, s)
+                      : chunk_launch<bf16_t>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, num_seqs, a, s);
+  return code;
 }
 
 KVF_EXPORT int kvf_mlstm_out(int dtype, const float* o, const void* g, int g_stride, const float* w, float eps,

@@ -123,6 +123,179 @@ __global__ __launch_bounds__(256) void moe_identity_kernel(float* __restrict__ x
   const T* hr = h + static_cast<size_t>(n) * width;
   for (int i = threadIdx.x; i < width; i += blockDim.x) xr[i] = fmaf(w, Elem<T>::load(hr + i), xr[i]);
 }
+
+// ---------------------------------------------------------------------------------------------
+// The experts' products over only the rows that chose them (bf16, matrix cores).
+//
+// moe_plan: the (token, choice) pairs are grouped by expert: where[pair] is the pair's place in
+// that order (-1 for a choice that names no expert), order[place] the pair; every expert's rows
+// are cut into tiles of 16: tiles[t] = (expert, first place, rows).  One workgroup; the order of
+// an expert's rows among themselves is whatever the atomics give, which no result depends on
+// (a row's products do not depend on its neighbours).
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+constexpr int TILE_ROWS = 16, PLAN_MAX_EXPERTS = 512;
+
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ sel, int pairs, int E,
+                                                        int* __restrict__ where, int* __restrict__ order,
+                                                        int* __restrict__ tiles, int* __restrict__ num_tiles,
+                                                        int max_tiles) {
+  __shared__ int cnt[PLAN_MAX_EXPERTS], off[PLAN_MAX_EXPERTS];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int p = tid; p < pairs; p += blockDim.x) {
+    const int e = sel[p];
+    where[p] = (e >= 0 && e < E) ? atomicAdd(&cnt[e], 1) : -1;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int o = 0, nt = 0;
+    for (int e = 0; e < E; ++e) {
+      off[e] = o;
+      const int c = cnt[e];
+      for (int r0 = 0; r0 < c && nt < max_tiles; r0 += TILE_ROWS) {
+        tiles[3 * nt] = e;
+        tiles[3 * nt + 1] = o + r0;
+        tiles[3 * nt + 2] = min(TILE_ROWS, c - r0);
+        ++nt;
+      }
+      o += c;
+    }
+    *num_tiles = nt;
+  }
+  __syncthreads();
+  for (int p = tid; p < pairs; p += blockDim.x) {
+    const int e = sel[p];
+    if (e >= 0 && e < E) {
+      const int pos = off[e] + where[p];
+      where[p] = pos;
+      order[pos] = p;
+    }
+  }
+}
+
+// v_mfma_f32_16x16x32_bf16 computes D[i][j] += sum_k A[i][k] B[j][k]; lane 16 c + r gives row r,
+// elements 8c..8c+7 of the step's 32 of either operand, and holds D[4 (l / 16) + v][l % 16].
+// A is a tile of the weight (1 KB in lane order, as ``StreamedWeight`` keeps it), B the tile's 16
+// rows: a lane ends with four neighbouring output columns of one row.
+//
+// moe_up: act[place, :] = silu(gate) * up for the tile's rows with their expert's matrices; the
+// weight holds every expert's gate and up rows interleaved (gate_j, up_j neighbours), so a lane's
+// four columns are two whole pairs.  Grid (column blocks, tiles); a wave takes GW groups of 16
+// weight rows.
+template <int GW>
+__global__ __launch_bounds__(256) void moe_up_kernel(const bf16_t* __restrict__ x, int ldx, int K,
+                                                     const uint4* __restrict__ wt, int S,
+                                                     const int* __restrict__ order,
+                                                     const int* __restrict__ tiles,
+                                                     const int* __restrict__ num_tiles, int top, int ff,
+                                                     bf16_t* __restrict__ act) {
+  const int tile = blockIdx.y;
+  if (tile >= *num_tiles) return;
+  const int e = tiles[3 * tile], row0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+  const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
+  const int j = lane % 16, c = lane / 16;
+  const int groups = ff / 8;   // groups of 16 interleaved rows per expert
+  const int g_first = (blockIdx.x * 4 + wave) * GW;
+  if (g_first >= groups) return;
+  const bf16_t* xr = j < rows ? x + static_cast<size_t>(order[row0 + j] / top) * ldx : nullptr;
+  f32x4 acc[GW];
+#pragma unroll
+  for (int g = 0; g < GW; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const uint4* wbase = wt + (static_cast<size_t>(e) * groups + g_first) * S * KVF_WAVE + lane;
+  for (int s = 0; s < S; ++s) {
+    uint4 xf = make_uint4(0u, 0u, 0u, 0u);
+    if (xr && 32 * s + 8 * c + 8 <= K) xf = *reinterpret_cast<const uint4*>(xr + 32 * s + 8 * c);
+    const bf16x8 b = __builtin_bit_cast(bf16x8, xf);
+#pragma unroll
+    for (int g = 0; g < GW; ++g) {
+      if (g_first + g < groups) {
+        const uint4 wf = wbase[(static_cast<size_t>(g) * S + s) * KVF_WAVE];
+        acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf), b, acc[g], 0, 0, 0);
+      }
+    }
+  }
+  if (j >= rows) return;
+  bf16_t* out = act + static_cast<size_t>(row0 + j) * ff;
+#pragma unroll
+  for (int g = 0; g < GW; ++g) {
+    if (g_first + g >= groups) continue;
+    const int col = (g_first + g) * 8 + 2 * c;
+    const float y0 = silu(acc[g][0]) * acc[g][1], y1 = silu(acc[g][2]) * acc[g][3];
+    *reinterpret_cast<uint32_t*>(out + col) =
+        static_cast<uint32_t>(f32_to_bf16(y0)) | (static_cast<uint32_t>(f32_to_bf16(y1)) << 16);
+  }
+}
+
+// moe_down: y[place, :] = act[place, :] W_down[expert]^T (bf16, not yet weighted).  The weight
+// holds the experts' down matrices side by side along K: expert e owns the steps e ff/32 ...
+template <int GW>
+__global__ __launch_bounds__(256) void moe_down_kernel(const bf16_t* __restrict__ act, int ff,
+                                                       const uint4* __restrict__ wt, int S_all,
+                                                       const int* __restrict__ tiles,
+                                                       const int* __restrict__ num_tiles,
+                                                       bf16_t* __restrict__ y, int hidden) {
+  const int tile = blockIdx.y;
+  if (tile >= *num_tiles) return;
+  const int e = tiles[3 * tile], row0 = tiles[3 * tile + 1], rows = tiles[3 * tile + 2];
+  const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE;
+  const int j = lane % 16, c = lane / 16;
+  const int groups = (hidden + 15) / 16;
+  const int g_first = (blockIdx.x * 4 + wave) * GW;
+  if (g_first >= groups) return;
+  const bf16_t* ar = j < rows ? act + static_cast<size_t>(row0 + j) * ff : nullptr;
+  f32x4 acc[GW];
+#pragma unroll
+  for (int g = 0; g < GW; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int S = ff / 32;
+  const uint4* wbase = wt + (static_cast<size_t>(g_first) * S_all + static_cast<size_t>(e) * S) * KVF_WAVE + lane;
+  for (int s = 0; s < S; ++s) {
+    uint4 af = make_uint4(0u, 0u, 0u, 0u);
+    if (ar) af = *reinterpret_cast<const uint4*>(ar + 32 * s + 8 * c);
+    const bf16x8 b = __builtin_bit_cast(bf16x8, af);
+#pragma unroll
+    for (int g = 0; g < GW; ++g) {
+      if (g_first + g < groups) {
+        const uint4 wf = wbase[(static_cast<size_t>(g) * S_all + s) * KVF_WAVE];
+        acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf), b, acc[g], 0, 0, 0);
+      }
+    }
+  }
+  if (j >= rows) return;
+  bf16_t* out = y + static_cast<size_t>(row0 + j) * hidden;
+#pragma unroll
+  for (int g = 0; g < GW; ++g) {
+    if (g_first + g >= groups) continue;
+    const int col = (g_first + g) * 16 + 4 * c;
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+      if (col + v < hidden) out[col + v].bits = f32_to_bf16(acc[g][v]);
+  }
+}
+
+// x[n, :] += sum over the token's choices, in their order, of weight * (the expert's row of y, or
+// the token's own input h for a choice that names no expert): fp32 sums into the fp32 stream.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, const bf16_t* __restrict__ y,
+                                                          const T* __restrict__ h, const int* __restrict__ sel,
+                                                          const float* __restrict__ wgt,
+                                                          const int* __restrict__ where, int hidden, int top,
+                                                          int E) {
+  const int n = blockIdx.x;
+  float* xr = x + static_cast<size_t>(n) * hidden;
+  const T* hr = h + static_cast<size_t>(n) * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int p = n * top + k, e = sel[p];
+      const float w = wgt[p];
+      if (e >= E) sum = fmaf(w, Elem<T>::load(hr + i), sum);
+      else if (e >= 0) sum = fmaf(w, bf16_to_f32(y[static_cast<size_t>(where[p]) * hidden + i].bits), sum);
+    }
+    xr[i] += sum;
+  }
+}
 }  // namespace
 
 KVF_EXPORT int kvf_moe_topk(const float* z, int z_stride, const float* correction, int* sel, float* wgt,
@@ -161,5 +334,41 @@ KVF_EXPORT int kvf_moe_identity(int dtype, float* x, const void* h, const int* s
                        sel, wgt, width, top, first);
   else
     return static_cast<int>(hipErrorInvalidValue);
+  return kvf_last_error();
+}
+
+// The routed experts of a bf16 step without the rows that did not choose them.  x [n, K] (row
+// stride ldx), w_gate_up / w_down: the tiled forms of [E 2 ff, K] (gate and up rows interleaved)
+// and [K, E ff]; sel / wgt [n, top]; scratch: where, order [n top], tiles [3 max_tiles],
+// num_tiles [1], act [n top, ff], y [n top, K].  Needs K % 8 == 0 and ff % 32 == 0.
+KVF_EXPORT int kvf_moe_grouped(const void* x, int ldx, const void* h, int n, int K, int E, int ff, int top,
+                               const void* w_gate_up, const void* w_down, const int* sel, const float* wgt,
+                               int* where, int* order, int* tiles, int* num_tiles, int max_tiles, void* act,
+                               void* y, float* residual, hipStream_t s) {
+  if (n <= 0) return 0;
+  const int pairs = n * top;
+  if (E <= 0 || E > PLAN_MAX_EXPERTS || K % 8 != 0 || ff % 32 != 0 || ldx % 8 != 0 || max_tiles > 65535 ||
+      max_tiles < (pairs + TILE_ROWS - 1) / TILE_ROWS + E)
+    return static_cast<int>(hipErrorInvalidValue);
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, s, sel, pairs, E, where, order, tiles, num_tiles,
+                     max_tiles);
+  const int S = (K + 31) / 32, up_groups = ff / 8, down_groups = (K + 15) / 16;
+  const bool many = pairs >= 1024;
+  const int gw = many ? 4 : 2;
+  const dim3 up_grid((up_groups + 4 * gw - 1) / (4 * gw), max_tiles), down_grid((down_groups + 4 * gw - 1) / (4 * gw), max_tiles);
+  const bf16_t* xb = static_cast<const bf16_t*>(x);
+  if (many) {
+    hipLaunchKernelGGL(moe_up_kernel<4>, up_grid, dim3(256), 0, s, xb, ldx, K, static_cast<const uint4*>(w_gate_up), S,
+                       order, tiles, num_tiles, top, ff, static_cast<bf16_t*>(act));
+    hipLaunchKernelGGL(moe_down_kernel<4>, down_grid, dim3(256), 0, s, static_cast<const bf16_t*>(act), ff,
+                       static_cast<const uint4*>(w_down), E * (ff / 32), tiles, num_tiles, static_cast<bf16_t*>(y), K);
+  } else {
+    hipLaunchKernelGGL(moe_up_kernel<2>, up_grid, dim3(256), 0, s, xb, ldx, K, static_cast<const uint4*>(w_gate_up), S,
+                       order, tiles, num_tiles, top, ff, static_cast<bf16_t*>(act));
+    hipLaunchKernelGGL(moe_down_kernel<2>, down_grid, dim3(256), 0, s, static_cast<const bf16_t*>(act), ff,
+                       static_cast<const uint4*>(w_down), E * (ff / 32), tiles, num_tiles, static_cast<bf16_t*>(y), K);
+  }
+  hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(n), dim3(256), 0, s, residual, static_cast<const bf16_t*>(y),
+                     static_cast<const bf16_t*>(h), sel, wgt, where, K, top, E);
   return kvf_last_error();
 }

@@ -1107,6 +1107,9 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
 
 
 # ------------------------------------------------------------------------------ matrix-memory recurrence
+MLSTM_CHUNK_FROM = 8     # runs of at least so many tokens go chunk by chunk on the matrix cores
+
+
 def mlstm_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
     """fp32 numbers of one request's state: per head the matrix ``[key_dim, value_dim]``, the
     normaliser ``[key_dim]`` and the running maximum."""
@@ -1116,16 +1119,21 @@ def mlstm_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
 def mlstm_scan(rows: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor, cu_q: torch.Tensor,
                positions: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor,
                num_seqs: int, heads: int, key_dim: int, value_dim: int, q_off: int, k_off: int,
-               v_off: int, cap: float, q_scale: float) -> None:
+               v_off: int, cap: float, q_scale: float, chunk_from: int = MLSTM_CHUNK_FROM,
+               short_runs: bool = True, long_runs: bool = True) -> None:
     """The matrix-memory recurrence over every sequence's tokens of this step, from and into the
     sequences' state slots.  ``rows [N, >= ...]``: projected rows holding q (``heads * key_dim``
     elements from column ``q_off``), k (from ``k_off``) and v (``heads * value_dim`` from
     ``v_off``); ``gates [N, 2 heads]`` fp32: input-gate then forget-gate pre-activations, to
-    which ``gate_bias [2 heads]`` is added before the cap ``cap * tanh(z / cap)``; the forget
+    (rows may be longer) which ``gate_bias [2 heads]`` is added before the cap ``cap * tanh(z / cap)``; the forget
     gate's log is ``logsigmoid`` of its capped value.  ``state [slots, mlstm_state_floats]``
     fp32; a sequence whose first token of the step sits at position 0 starts from zeros whatever
     its slot holds; a negative slot skips the sequence.  ``out [N, heads * value_dim]`` fp32: the
-    heads' outputs ``S^T q / (max(|n . q|, exp(-m)) + 1e-6)`` with ``q`` times ``q_scale``."""
+    heads' outputs ``S^T q / (max(|n . q|, exp(-m)) + 1e-6)`` with ``q`` times ``q_scale``.
+    Two kernels share the work: runs of fewer than ``chunk_from`` tokens are walked token by
+    token, longer ones a chunk at a time on the matrix cores (in fp32); ``short_runs`` /
+    ``long_runs`` say which of the two are launched (a caller that knows its runs' lengths
+    spares the other launch)."""
     n = rows.shape[0]
     H, dk, dv = int(heads), int(key_dim), int(value_dim)
     _check(rows, "rows", None, (n, None), contiguous=False)
@@ -1136,7 +1144,9 @@ def mlstm_scan(rows: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor,
             raise KernelError(f"mlstm_scan: {name} at columns {off}..{off + size} lies outside rows of {rows.shape[1]}")
     if not 0 < dk <= 256:
         raise KernelError(f"mlstm_scan: key sizes up to 256, got {dk}")
-    _check(gates, "gates", F32, (n, 2 * H))
+    _check(gates, "gates", F32, (n, None))
+    if gates.shape[1] < 2 * H:
+        raise KernelError(f"mlstm_scan: gate rows of {gates.shape[1]} numbers do not hold {2 * H} gates")
     _check(gate_bias, "gate_bias", F32, (2 * H,))
     _check(cu_q, "cu_q", I32, (None,))
     _check(positions, "positions", I32, (None,))
@@ -1145,11 +1155,14 @@ def mlstm_scan(rows: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor,
         raise KernelError("mlstm_scan: cu_q / slot_ids / positions shorter than the batch")
     _check(state, "state", F32, (None, mlstm_state_floats(H, dk, dv)))
     _check(out, "out", F32, (n, H * dv))
-    f = _fn("mlstm", "kvf_mlstm_scan", [c_int] + [c_void_p] * 8 + [c_int] * 9 + [c_float, c_float, c_void_p])
+    if chunk_from < 1:
+        raise KernelError(f"mlstm_scan: chunk_from must be positive, got {chunk_from}")
+    f = _fn("mlstm", "kvf_mlstm_scan", [c_int] + [c_void_p] * 8 + [c_int] * 10 + [c_float, c_float] + [c_int] * 3 + [c_void_p])
     _ok(f(_tcode(rows.dtype), rows.data_ptr(), gates.data_ptr(), gate_bias.data_ptr(), cu_q.data_ptr(),
           positions.data_ptr(), slot_ids.data_ptr(), state.data_ptr(), out.data_ptr(), int(num_seqs),
           H, dk, dv, rows.stride(0) if n > 1 else rows.shape[1], int(q_off), int(k_off), int(v_off),
-          state.shape[0], float(cap), float(q_scale), _stream()), "mlstm_scan")
+          state.shape[0], gates.shape[1], float(cap), float(q_scale), int(chunk_from), 1 if short_runs else 0,
+          1 if long_runs else 0, _stream()), "mlstm_scan")
 
 
 def mlstm_out(heads_raw: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float,
@@ -1226,6 +1239,54 @@ def moe_identity(x: torch.Tensor, h: torch.Tensor, chosen: torch.Tensor, weights
     f = _fn("moe", "kvf_moe_identity", [c_int] + [c_void_p] * 4 + [c_int] * 4 + [c_void_p])
     _ok(f(_tcode(h.dtype), x.data_ptr(), h.data_ptr(), chosen.data_ptr(), weights.data_ptr(), n, width,
           top, int(first), _stream()), "moe_identity")
+
+
+def moe_grouped_takes(x: torch.Tensor, w_gate_up, w_down, experts: int, ff: int) -> bool:
+    """Whether ``moe_grouped`` takes these operands: bf16 rows that start on 16 bytes, both
+    weights kept in tiles, a width that is a multiple of 8 and experts whose width is a
+    multiple of 32."""
+    n, k = x.shape
+    return (x.dtype == BF16 and isinstance(w_gate_up, StreamedWeight) and isinstance(w_down, StreamedWeight)
+            and _rows_aligned(x, k, x.stride(0) if n > 1 else k) and ff % 32 == 0 and 0 < experts <= 512)
+
+
+def moe_grouped_tiles(rows: int, top: int, experts: int) -> int:
+    """Tiles of 16 rows that the (token, choice) pairs of ``rows`` tokens can make at most."""
+    return -(-rows * top // 16) + experts
+
+
+def moe_grouped(x: torch.Tensor, w_gate_up: "StreamedWeight", w_down: "StreamedWeight", chosen: torch.Tensor,
+                weights: torch.Tensor, residual: torch.Tensor, experts: int, ff: int,
+                scratch: dict[str, torch.Tensor]) -> None:
+    """``residual[n] += sum_k weights[n, k] * expert_{chosen[n, k]}(x[n])`` (a choice ``>= experts``
+    stands for ``x[n]`` itself) with every expert's products taken over only the rows that chose
+    it: the pairs are grouped by expert on the device, tiles of 16 rows go through the
+    matrix cores against the expert's tiles of ``w_gate_up`` (``[experts * 2 ff, K]``, gate and
+    up rows interleaved) and ``w_down`` (``[K, experts * ff]``), an expert's output row is stored
+    in bf16 and the weighted sum over a token's choices is taken in fp32 in their order.
+    ``scratch``: ``where order [n top]``, ``tiles [3 moe_grouped_tiles]``, ``num_tiles [1]`` (int32),
+    ``act [n top, ff]``, ``y [n top, K]`` (bf16)."""
+    n, k = x.shape
+    top = chosen.shape[1]
+    if not moe_grouped_takes(x, w_gate_up, w_down, experts, ff):
+        raise KernelError("moe_grouped: operands it does not take (see moe_grouped_takes)")
+    if tuple(w_gate_up.shape) != (experts * 2 * ff, k) or tuple(w_down.shape) != (k, experts * ff):
+        raise KernelError(f"moe_grouped: weights {list(w_gate_up.shape)} / {list(w_down.shape)} do not fit "
+                          f"{experts} experts of width {ff} over rows of {k}")
+    _check(chosen, "chosen", I32, (n, top))
+    _check(weights, "weights", F32, (n, top))
+    _check(residual, "residual", F32, (n, k))
+    pairs, max_tiles = n * top, moe_grouped_tiles(n, top, experts)
+    for name, dtype, shape in (("where", I32, (pairs,)), ("order", I32, (pairs,)), ("tiles", I32, (3 * max_tiles,)),
+                               ("num_tiles", I32, (1,)), ("act", BF16, (pairs, ff)), ("y", BF16, (pairs, k))):
+        _check(scratch[name], name, dtype, shape)
+    f = _fn("moe", "kvf_moe_grouped", [c_void_p, c_int, c_void_p] + [c_int] * 5 + [c_void_p] * 8 + [c_int]
+            + [c_void_p] * 4)
+    _ok(f(x.data_ptr(), x.stride(0) if n > 1 else k, x.data_ptr(), n, k, int(experts), int(ff), top,
+          w_gate_up.tiles.data_ptr(), w_down.tiles.data_ptr(), chosen.data_ptr(), weights.data_ptr(),
+          scratch["where"].data_ptr(), scratch["order"].data_ptr(), scratch["tiles"].data_ptr(),
+          scratch["num_tiles"].data_ptr(), max_tiles, scratch["act"].data_ptr(), scratch["y"].data_ptr(),
+          residual.data_ptr(), _stream()), "moe_grouped")
 
 
 # ------------------------------------------------------------------------------ sampling

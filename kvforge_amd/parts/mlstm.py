@@ -65,28 +65,34 @@ class MatrixLSTM(Mixer):
             mats = [m.float() for m in mats]
         # one product for q, k, v and the output gate: their heads side by side in that order
         self.w_rows = torch.cat(mats, dim=0).contiguous()
-        # the gates' product is held in fp32, so that it runs the 32-bit kernel and its sums are
-        # stored unrounded
-        self.w_gates = torch.cat([t("i"), t("f")], dim=0).float().contiguous()
+        # the gates' product: input gates' rows, then forget gates', padded with zero rows to a
+        # multiple of 16 (which every product kernel takes); its 32-bit sums are stored in fp32
+        gi, gf = t("i"), t("f")
+        if gi.dtype != gf.dtype:
+            gi, gf = gi.float(), gf.float()
+        self.G_pad = -(-2 * self.H // 16) * 16
+        self.w_gates = torch.cat([gi, gf, gi.new_zeros(self.G_pad - 2 * self.H, self.hidden)], dim=0).contiguous()
         self.gate_bias = torch.cat([t("i", self.bias_suffix), t("f", self.bias_suffix)], dim=0).float().contiguous()
         self.head_weight = t("norm").float().contiguous()
         self.w_o = t("o")
 
     def seal(self) -> None:
         self.w_rows, self.w_o = ops.streamed(ops.plain_of(self.w_rows)), ops.streamed(ops.plain_of(self.w_o))
+        self.w_gates = ops.streamed(ops.plain_of(self.w_gates))
 
     def kernel_modules(self, dtype: torch.dtype) -> set[str]:
         return {"mlstm", "gemm_generic"} | ({"gemm_bf16"} if dtype == torch.bfloat16 else set())
 
     def _small(self) -> list[torch.Tensor]:
-        return [x for x in (self.w_gates, self.gate_bias, self.head_weight) if x is not None]
+        return [x for x in (ops.plain_of(self.w_gates), self.gate_bias, self.head_weight) if x is not None]
 
     def num_bytes(self) -> int:
         return sum(x.numel() * x.element_size()
                    for x in (*map(ops.plain_of, (self.w_rows, self.w_o)), *self._small()) if x is not None)
 
     def held_tensors(self) -> list[torch.Tensor]:
-        return ops.copies_of(self.w_rows) + ops.copies_of(self.w_o) + self._small()
+        return (ops.copies_of(self.w_rows) + ops.copies_of(self.w_o) + ops.copies_of(self.w_gates)
+                + [x for x in (self.gate_bias, self.head_weight) if x is not None])
 
     def forward(self, x, step, layer: LayerState, residual) -> None:
         """``x``: normalised activations."""
@@ -98,12 +104,16 @@ class MatrixLSTM(Mixer):
         step.settle()
         rows = ws.buf("mlstm_rows", (n, 2 * H * dk + 2 * H * dv), act)
         ops.gemm(x, self.w_rows, rows)
-        gates = ws.buf("mlstm_gates", (n, 2 * H), torch.float32)
+        gates = ws.buf("mlstm_gates", (n, self.G_pad), torch.float32)
         ops.gemm(x, self.w_gates, gates)
         raw = ws.buf("mlstm_raw", (n, H * dv), torch.float32)
+        # which of the two kernels have work is known from the runs' lengths (all ones in a
+        # captured step of single tokens, so a replay launches what the capture launched)
+        long_runs = any(q >= ops.MLSTM_CHUNK_FROM for q in step.q_lens)
+        short_runs = any(q < ops.MLSTM_CHUNK_FROM for q in step.q_lens)
         ops.mlstm_scan(rows, gates, self.gate_bias, step.cu_q, step.positions, step.slot_ids,
                        layer.state, raw, step.n_seqs, H, dk, dv, 0, H * dk, 2 * H * dk,
-                       self.gate_cap, float(dk) ** -0.5)
+                       self.gate_cap, float(dk) ** -0.5, short_runs=short_runs, long_runs=long_runs)
         heads = ws.buf("mlstm_heads", (n, H * dv), act)
         g0 = 2 * H * dk + H * dv
         ops.mlstm_out(raw, rows[:, g0:g0 + H * dv], self.head_weight, self.norm_eps, heads, H, dv)

@@ -61,7 +61,12 @@ class RoutedExperts(FeedForward):
         return out
 
     def load(self, tensors: dict[str, torch.Tensor]) -> None:
-        self.w_router = tensors[self._name(self.names["router"])].float().contiguous()
+        # the router's rows padded with zero rows to a multiple of 16, which every product kernel
+        # takes; in the engine's type: products of bfloat16 numbers are exact in 32 bits, and the
+        # sums are 32-bit and stored so
+        r = tensors[self._name(self.names["router"])]
+        self.R_pad = -(-self.R // 16) * 16
+        self.w_router = torch.cat([r, r.new_zeros(self.R_pad - self.R, self.hidden)], dim=0).contiguous()
         self.correction = tensors[self._name(self.names["correction"])].float().contiguous()
         pairs, downs = [], []
         for e in range(self.E):
@@ -82,6 +87,7 @@ class RoutedExperts(FeedForward):
     def seal(self) -> None:
         self.w_gate_up = ops.streamed(ops.plain_of(self.w_gate_up))
         self.w_down = ops.streamed(ops.plain_of(self.w_down))
+        self.w_router = ops.streamed(ops.plain_of(self.w_router))
         if self.shared is not None:
             self.shared.seal()
 
@@ -94,13 +100,14 @@ class RoutedExperts(FeedForward):
         the shared expert."""
         experts = sum(t.numel() * t.element_size() for t in map(ops.plain_of, (self.w_gate_up, self.w_down))
                       if t is not None)
-        small = sum(t.numel() * t.element_size() for t in (self.w_router, self.correction) if t is not None)
+        small = sum(t.numel() * t.element_size() for t in (ops.plain_of(self.w_router), self.correction)
+                    if t is not None)
         return (small + experts * min(self.top, self.E) // max(self.E, 1)
                 + (self.shared.num_bytes() if self.shared is not None else 0))
 
     def held_tensors(self) -> list[torch.Tensor]:
         return (ops.copies_of(self.w_gate_up) + ops.copies_of(self.w_down)
-                + [t for t in (self.w_router, self.correction) if t is not None]
+                + ops.copies_of(self.w_router) + ([self.correction] if self.correction is not None else [])
                 + (self.shared.held_tensors() if self.shared is not None else []))
 
     def forward(self, x, step, residual) -> None:
@@ -108,11 +115,26 @@ class RoutedExperts(FeedForward):
         n = x.shape[0]
         ws, dt = step.ws, step.act_dtype
         step.settle()
-        logits = ws.buf("moe_logits", (n, self.R), torch.float32)
-        ops.gemm(x, self.w_router, logits)          # a 32-bit product: the router's matrix is fp32
+        logits = ws.buf("moe_logits", (n, self.R_pad), torch.float32)[:, :self.R]
+        ops.gemm(x, self.w_router, ws.buf("moe_logits", (n, self.R_pad), torch.float32))   # 32-bit sums, stored so
         chosen = ws.buf("moe_chosen", (n, self.top), torch.int32)
         weights = ws.buf("moe_weights", (n, self.top), torch.float32)
         ops.moe_topk(logits, self.correction, chosen, weights)
+        if ops.moe_grouped_takes(x, self.w_gate_up, self.w_down, self.E, self.ff) and x.is_contiguous():
+            # bf16: every expert over only the rows that chose it, grouped on the device
+            pairs, tiles = n * self.top, ops.moe_grouped_tiles(n, self.top, self.E)
+            scratch = {"where": ws.buf("moe_where", (pairs,), torch.int32),
+                       "order": ws.buf("moe_order", (pairs,), torch.int32),
+                       "tiles": ws.buf("moe_tiles", (3 * tiles,), torch.int32),
+                       "num_tiles": ws.buf("moe_num_tiles", (1,), torch.int32),
+                       "act": ws.buf("moe_act_rows", (pairs, self.ff), dt),
+                       "y": ws.buf("moe_y_rows", (pairs, self.hidden), dt)}
+            ops.moe_grouped(x, self.w_gate_up, self.w_down, chosen, weights, residual, self.E, self.ff, scratch)
+            if self.shared is not None:
+                self.shared.forward(x, step, residual)
+            return
+        # otherwise (32-bit, or sizes the grouped kernels do not take): every expert over every
+        # row in one product, the rows that did not choose it multiplied by an exact zero
         if self.identity:
             ops.moe_identity(residual, x, chosen, weights, self.E)
         gu = ws.buf("moe_gate_up", (n, 2 * self.E * self.ff), dt)

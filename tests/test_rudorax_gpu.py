@@ -164,10 +164,13 @@ def scan_reference(q, k, v, zi, zf, bias, cap, H, dk, dv):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,dk,dv", [(2, 8, 16), (6, 32, 64), (1, 40, 100), (3, 64, 24), (2, 100, 130),
                                      (2, 128, 64), (1, 200, 70), (1, 256, 8)])
-def test_matrix_memory_over_runs_and_steps(dtype, H, dk, dv):
+@pytest.mark.parametrize("chunk_from", [1, 8, 1000])
+def test_matrix_memory_over_runs_and_steps(dtype, H, dk, dv, chunk_from):
     """Four sequences in three steps: runs of many tokens, of two and of one; a sequence that
     starts in the slot another gave back (which still holds that one's state); a sequence
-    without a slot.  Gates reach both ends of their cap."""
+    without a slot.  Gates reach both ends of their cap.  ``chunk_from``: every run chunk by
+    chunk on the matrix cores, every run token by token, and the two kernels side by side in
+    one step, each carrying on from the state the other left."""
     cap = 6.0
     lens = {"a": 23, "b": 9, "c": 1, "d": 12}
     cols = 2 * H * dk + H * dv + 5                      # rows wider than q, k, v: something behind them
@@ -193,7 +196,7 @@ def test_matrix_memory_over_runs_and_steps(dtype, H, dk, dv):
         pos = torch.cat([torch.arange(a, b) for _, a, b in step] + [torch.zeros(1, dtype=torch.long)]).int().to(DEV)
         out = torch.full((rows.shape[0], H * dv), 5.0, device=DEV)
         ops().mlstm_scan(rows, z, bias.to(DEV), cu, pos, i32([slot[r] for r, _, _ in step] + [-1]), state, out,
-                         len(counts), H, dk, dv, 0, H * dk, 2 * H * dk, cap, dk ** -0.5)
+                         len(counts), H, dk, dv, 0, H * dk, 2 * H * dk, cap, dk ** -0.5, chunk_from=chunk_from)
         off = 0
         for (r, a, b) in step:
             got[r].append(out[off:off + b - a].cpu())
@@ -201,6 +204,30 @@ def test_matrix_memory_over_runs_and_steps(dtype, H, dk, dv):
         assert float(out[off:].abs().max()) == 0.0       # the sequence without a slot
     for r in lens:
         torch.testing.assert_close(torch.cat(got[r]), want[r], atol=2e-4, rtol=2e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,dk,dv", [(2, 40, 72), (1, 136, 64), (1, 256, 40), (3, 16, 130)])
+def test_matrix_memory_over_many_chunks(dtype, H, dk, dv):
+    """A run of 203 tokens in portions that end inside chunks, the state handed from chunk to
+    chunk and from step to step; forget gates that stay open, so that the first tokens still
+    weigh at the end."""
+    cap, T = 15.0, 203
+    cols = 2 * H * dk + H * dv
+    rows, z = rand(T, cols, seed=dk).to(dtype), rand(T, 2 * H, seed=dv, scale=3.0)
+    bias = torch.cat([torch.full((H,), -1.0), torch.full((H,), 6.0)])
+    x = rows.float()
+    want = scan_reference(x[:, :H * dk], x[:, H * dk:2 * H * dk], x[:, 2 * H * dk:], z[:, :H], z[:, H:], bias, cap, H, dk, dv)
+    state = torch.full((2, ops().mlstm_state_floats(H, dk, dv)), 3.0, device=DEV)
+    got = []
+    for a, b in ((0, 130), (130, 131), (131, 203)):
+        out = torch.empty(b - a, H * dv, device=DEV)
+        ops().mlstm_scan(rows[a:b].to(DEV), z[a:b].to(DEV), bias.to(DEV), i32([0, b - a]),
+                         torch.arange(a, b, dtype=torch.int32, device=DEV), i32([1]), state, out, 1, H, dk, dv,
+                         0, H * dk, 2 * H * dk, cap, dk ** -0.5)
+        got.append(out.cpu())
+    torch.testing.assert_close(torch.cat(got), want, atol=3e-4, rtol=3e-4)
+    assert float(state[0].min()) == 3.0                       # the other slot is nobody's business
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -231,10 +258,13 @@ def test_router_chooses_by_corrected_probability_and_weighs_by_probability(R, to
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("n", [1, 5, 70])
-@pytest.mark.parametrize("E,I,top,ff,shared", [(4, 0, 1, 16, 0), (16, 4, 3, 24, 40), (5, 2, 7, 8, 16), (8, 1, 2, 72, 0)])
+@pytest.mark.parametrize("n", [1, 5, 70, 300])
+@pytest.mark.parametrize("E,I,top,ff,shared", [(4, 0, 1, 16, 0), (16, 4, 3, 24, 40), (5, 2, 7, 8, 16), (8, 1, 2, 72, 0),
+                                               (6, 2, 3, 32, 16), (33, 0, 4, 64, 0), (3, 1, 2, 96, 8)])
 def test_routed_feed_forward_alone(dtype, n, E, I, top, ff, shared):
-    """The part by itself on a step of ``n`` rows: few rows and many take other products."""
+    """The part by itself on a step of ``n`` rows: few rows and many take other products; expert
+    widths that are a multiple of 32 take the grouped kernels in bfloat16, the others (and
+    32-bit) the product over all experts."""
     from kvforge_amd.engine.batch import Step, Workspace
     from kvforge_amd.parts import RoutedExperts
     h = 48
