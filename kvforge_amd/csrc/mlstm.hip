@@ -162,11 +162,11 @@ __global__ __launch_bounds__(ROWS > KVF_WAVE ? 2 * KVF_WAVE : KVF_WAVE) void mls
 //   D[t][s] = exp(b_t - b_s + li_s - m_t) for s <= t (0 otherwise),  g_t = exp(b_t + m_c - m_t)
 //   A = (Q K^T) * D;   O = A V + diag(g) Q S;   n_t . q_t = rowsum(A)_t + g_t q_t . n
 //   S' = g_L S + K^T diag(D[L]) V;   n' = g_L n + K^T D[L];   m_c' = m_L        (L: the last token)
-// which is the recurrence written out over the chunk.  A workgroup of four waves takes 64 columns
+// which is the recurrence written out over the chunk.  A workgroup of four waves takes 32 columns
 // of S for one (sequence, head); Q, K (fp32, rows padded to an odd stride), the V columns, A and
 // the S columns live in LDS.
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-constexpr int CCOLS = 64;
+constexpr int CCOLS = 32;
 
 template <typename T, int DKP, int CL>
 __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ qkv, const float* __restrict__ zif,
@@ -238,34 +238,44 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
                   ? Elem<T>::load(qkv + static_cast<size_t>(tb + t) * a.row_len + a.v_off + head * dv + c)
                   : 0.f;
     }
-    if (tid < CL) {
+    if (wave == 0) {
+      // a lane per token: the gates, the running sum of the log forget gates (64-bit) and the
+      // running maximum, which the recurrence m_t = max(lf_t + m_(t-1), li_t) gives as
+      // m_t = b_t + max(m_c, max over s <= t of (li_s - b_s)): two scans over the wave
+      const int t = lane;
       float i_gate = 0.f, f_gate = 0.f;
-      if (tid < cnt) {
-        const float* z = zif + static_cast<size_t>(tb + tid) * a.gate_stride;
+      if (t < cnt) {
+        const float* z = zif + static_cast<size_t>(tb + t) * a.gate_stride;
         i_gate = capped(z[head] + bias_if[head], a.cap);
         f_gate = log_sigmoid(capped(z[a.H + head] + bias_if[a.H + head], a.cap));
       }
-      li[tid] = i_gate;
-      bc[tid] = static_cast<double>(f_gate);
-    }
-    __syncthreads();
-    if (tid == 0) {   // the recurrence of the maximum, token by token, and the gates' running sum
-      float m = m_c;
-      double b = 0.0;
-      for (int t = 0; t < cnt; ++t) {
-        const float f = static_cast<float>(bc[t]);
-        m = fmaxf(f + m, li[t]);
-        b += static_cast<double>(f);
+      double b = static_cast<double>(f_gate);
+#pragma unroll
+      for (int o = 1; o < KVF_WAVE; o <<= 1) {
+        const double up = __shfl_up(b, o, KVF_WAVE);
+        if (lane >= o) b += up;
+      }
+      double u = t < cnt ? static_cast<double>(i_gate) - b : -1e300;
+#pragma unroll
+      for (int o = 1; o < KVF_WAVE; o <<= 1) {
+        const double up = __shfl_up(u, o, KVF_WAVE);
+        if (lane >= o) u = fmax(u, up);
+      }
+      const float mc = m_c;
+      const float m = static_cast<float>(b + fmax(static_cast<double>(mc), u));
+      const int last_t = cnt - 1;
+      const double b_last = __shfl(b, last_t, KVF_WAVE);
+      const float m_last = __shfl(m, last_t, KVF_WAVE);
+      if (t < CL) {
+        li[t] = i_gate;
         bc[t] = b;
-        mt[t] = m;
+        mt[t] = t < cnt ? m : m_last;
+        gt[t] = t < cnt ? expf(static_cast<float>(b + static_cast<double>(mc) - static_cast<double>(m))) : 0.f;
+        wl[t] = t < cnt ? expf(static_cast<float>(b_last - b) + i_gate - m_last) : 0.f;
       }
     }
     __syncthreads();
     const int last = cnt - 1;
-    if (tid < CL) {
-      gt[tid] = tid < cnt ? expf(static_cast<float>(bc[tid] + static_cast<double>(m_c) - static_cast<double>(mt[tid]))) : 0.f;
-      wl[tid] = tid < cnt ? expf(static_cast<float>(bc[last] - bc[tid]) + li[tid] - mt[last]) : 0.f;
-    }
     // ---- A = (Q K^T) * D, tile by tile; tiles above the diagonal are zero
     constexpr int RT = CL / 16;
     for (int tile = wave; tile < RT * RT; tile += 4) {

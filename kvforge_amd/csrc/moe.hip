@@ -129,17 +129,17 @@ __global__ __launch_bounds__(256) void moe_identity_kernel(float* __restrict__ x
 //
 // moe_plan: the (token, choice) pairs are grouped by expert: where[pair] is the pair's place in
 // that order (-1 for a choice that names no expert), order[place] the pair; every expert's rows
-// are cut into tiles of 16: tiles[t] = (expert, first place, rows).  One workgroup; the order of
+// are cut into tiles of tile_rows: tiles[t] = (expert, first place, rows).  One workgroup; the order of
 // an expert's rows among themselves is whatever the atomics give, which no result depends on
 // (a row's products do not depend on its neighbours).
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
-constexpr int TILE_ROWS = 16, PLAN_MAX_EXPERTS = 512;
+constexpr int PLAN_MAX_EXPERTS = 512;
 
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ sel, int pairs, int E,
                                                         int* __restrict__ where, int* __restrict__ order,
                                                         int* __restrict__ tiles, int* __restrict__ num_tiles,
-                                                        int max_tiles) {
+                                                        int max_tiles, int tile_rows) {
   __shared__ int cnt[PLAN_MAX_EXPERTS], off[PLAN_MAX_EXPERTS];
   const int tid = threadIdx.x;
   for (int e = tid; e < E; e += blockDim.x) cnt[e] = 0;
@@ -154,10 +154,10 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
     for (int e = 0; e < E; ++e) {
       off[e] = o;
       const int c = cnt[e];
-      for (int r0 = 0; r0 < c && nt < max_tiles; r0 += TILE_ROWS) {
+      for (int r0 = 0; r0 < c && nt < max_tiles; r0 += tile_rows) {
         tiles[3 * nt] = e;
         tiles[3 * nt + 1] = o + r0;
-        tiles[3 * nt + 2] = min(TILE_ROWS, c - r0);
+        tiles[3 * nt + 2] = min(tile_rows, c - r0);
         ++nt;
       }
       o += c;
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ 
 // weight holds every expert's gate and up rows interleaved (gate_j, up_j neighbours), so a lane's
 // four columns are two whole pairs.  Grid (column blocks, tiles); a wave takes GW groups of 16
 // weight rows.
-template <int GW>
+template <int RT, int GW>
 __global__ __launch_bounds__(256) void moe_up_kernel(const bf16_t* __restrict__ x, int ldx, int K,
                                                      const uint4* __restrict__ wt, int S,
                                                      const int* __restrict__ order,
@@ -199,38 +199,59 @@ __global__ __launch_bounds__(256) void moe_up_kernel(const bf16_t* __restrict__ 
   const int groups = ff / 8;   // groups of 16 interleaved rows per expert
   const int g_first = (blockIdx.x * 4 + wave) * GW;
   if (g_first >= groups) return;
-  const bf16_t* xr = j < rows ? x + static_cast<size_t>(order[row0 + j] / top) * ldx : nullptr;
-  f32x4 acc[GW];
+  // a tile holds RT sub-tiles of 16 rows; a weight fragment is loaded once for all of them
+  const bf16_t* xr[RT];
 #pragma unroll
-  for (int g = 0; g < GW; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < RT; ++r)
+    xr[r] = 16 * r + j < rows ? x + static_cast<size_t>(order[row0 + 16 * r + j] / top) * ldx + 8 * c : nullptr;
+  f32x4 acc[RT][GW];
+#pragma unroll
+  for (int r = 0; r < RT; ++r)
+#pragma unroll
+    for (int g = 0; g < GW; ++g) acc[r][g] = f32x4{0.f, 0.f, 0.f, 0.f};
   const uint4* wbase = wt + (static_cast<size_t>(e) * groups + g_first) * S * KVF_WAVE + lane;
-  for (int s = 0; s < S; ++s) {
-    uint4 xf = make_uint4(0u, 0u, 0u, 0u);
-    if (xr && 32 * s + 8 * c + 8 <= K) xf = *reinterpret_cast<const uint4*>(xr + 32 * s + 8 * c);
-    const bf16x8 b = __builtin_bit_cast(bf16x8, xf);
+  const int s_full = K / 32;   // steps whose 32 elements all lie inside a row
+  auto step = [&](int s) {
+    bf16x8 b[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      uint4 xf = make_uint4(0u, 0u, 0u, 0u);
+      if (xr[r] && (s < s_full || 32 * s + 8 * c + 8 <= K)) xf = *reinterpret_cast<const uint4*>(xr[r] + 32 * s);
+      b[r] = __builtin_bit_cast(bf16x8, xf);
+    }
+#pragma unroll
+    for (int g = 0; g < GW; ++g) {   // ff is a multiple of 32, so the groups come in whole fours
+      const bf16x8 wf = __builtin_bit_cast(bf16x8, wbase[(static_cast<size_t>(g) * S + s) * KVF_WAVE]);
+#pragma unroll
+      for (int r = 0; r < RT; ++r) acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, b[r], acc[r][g], 0, 0, 0);
+    }
+  };
+  int s = 0;
+  for (; s + 4 <= S; s += 4) {
+    step(s);
+    step(s + 1);
+    step(s + 2);
+    step(s + 3);
+  }
+  for (; s < S; ++s) step(s);
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    if (16 * r + j >= rows) continue;
+    bf16_t* out = act + static_cast<size_t>(row0 + 16 * r + j) * ff;
 #pragma unroll
     for (int g = 0; g < GW; ++g) {
-      if (g_first + g < groups) {
-        const uint4 wf = wbase[(static_cast<size_t>(g) * S + s) * KVF_WAVE];
-        acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf), b, acc[g], 0, 0, 0);
-      }
+      if (g_first + g >= groups) continue;
+      const int col = (g_first + g) * 8 + 2 * c;
+      const float y0 = silu(acc[r][g][0]) * acc[r][g][1], y1 = silu(acc[r][g][2]) * acc[r][g][3];
+      *reinterpret_cast<uint32_t*>(out + col) =
+          static_cast<uint32_t>(f32_to_bf16(y0)) | (static_cast<uint32_t>(f32_to_bf16(y1)) << 16);
     }
-  }
-  if (j >= rows) return;
-  bf16_t* out = act + static_cast<size_t>(row0 + j) * ff;
-#pragma unroll
-  for (int g = 0; g < GW; ++g) {
-    if (g_first + g >= groups) continue;
-    const int col = (g_first + g) * 8 + 2 * c;
-    const float y0 = silu(acc[g][0]) * acc[g][1], y1 = silu(acc[g][2]) * acc[g][3];
-    *reinterpret_cast<uint32_t*>(out + col) =
-        static_cast<uint32_t>(f32_to_bf16(y0)) | (static_cast<uint32_t>(f32_to_bf16(y1)) << 16);
   }
 }
 
 // moe_down: y[place, :] = act[place, :] W_down[expert]^T (bf16, not yet weighted).  The weight
 // holds the experts' down matrices side by side along K: expert e owns the steps e ff/32 ...
-template <int GW>
+template <int RT, int GW>
 __global__ __launch_bounds__(256) void moe_down_kernel(const bf16_t* __restrict__ act, int ff,
                                                        const uint4* __restrict__ wt, int S_all,
                                                        const int* __restrict__ tiles,
@@ -244,33 +265,55 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const bf16_t* __restrict_
   const int groups = (hidden + 15) / 16;
   const int g_first = (blockIdx.x * 4 + wave) * GW;
   if (g_first >= groups) return;
-  const bf16_t* ar = j < rows ? act + static_cast<size_t>(row0 + j) * ff : nullptr;
-  f32x4 acc[GW];
+  const bf16_t* ar[RT];
 #pragma unroll
-  for (int g = 0; g < GW; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int r = 0; r < RT; ++r)
+    ar[r] = 16 * r + j < rows ? act + static_cast<size_t>(row0 + 16 * r + j) * ff + 8 * c : nullptr;
+  f32x4 acc[RT][GW];
+#pragma unroll
+  for (int r = 0; r < RT; ++r)
+#pragma unroll
+    for (int g = 0; g < GW; ++g) acc[r][g] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int S = ff / 32;
   const uint4* wbase = wt + (static_cast<size_t>(g_first) * S_all + static_cast<size_t>(e) * S) * KVF_WAVE + lane;
-  for (int s = 0; s < S; ++s) {
-    uint4 af = make_uint4(0u, 0u, 0u, 0u);
-    if (ar) af = *reinterpret_cast<const uint4*>(ar + 32 * s + 8 * c);
-    const bf16x8 b = __builtin_bit_cast(bf16x8, af);
+  int goff[GW];
+#pragma unroll
+  for (int g = 0; g < GW; ++g) goff[g] = min(g, groups - 1 - g_first);
+  auto step = [&](int s) {
+    bf16x8 b[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      uint4 af = make_uint4(0u, 0u, 0u, 0u);
+      if (ar[r]) af = *reinterpret_cast<const uint4*>(ar[r] + 32 * s);
+      b[r] = __builtin_bit_cast(bf16x8, af);
+    }
+#pragma unroll
+    for (int g = 0; g < GW; ++g) {   // a group past the last is read as the last and not stored
+      const bf16x8 wf = __builtin_bit_cast(bf16x8, wbase[(static_cast<size_t>(goff[g]) * S_all + s) * KVF_WAVE]);
+#pragma unroll
+      for (int r = 0; r < RT; ++r) acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, b[r], acc[r][g], 0, 0, 0);
+    }
+  };
+  int s = 0;
+  for (; s + 4 <= S; s += 4) {
+    step(s);
+    step(s + 1);
+    step(s + 2);
+    step(s + 3);
+  }
+  for (; s < S; ++s) step(s);
+#pragma unroll
+  for (int r = 0; r < RT; ++r) {
+    if (16 * r + j >= rows) continue;
+    bf16_t* out = y + static_cast<size_t>(row0 + 16 * r + j) * hidden;
 #pragma unroll
     for (int g = 0; g < GW; ++g) {
-      if (g_first + g < groups) {
-        const uint4 wf = wbase[(static_cast<size_t>(g) * S_all + s) * KVF_WAVE];
-        acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wf), b, acc[g], 0, 0, 0);
-      }
+      if (g_first + g >= groups) continue;
+      const int col = (g_first + g) * 16 + 4 * c;
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        if (col + v < hidden) out[col + v].bits = f32_to_bf16(acc[r][g][v]);
     }
-  }
-  if (j >= rows) return;
-  bf16_t* out = y + static_cast<size_t>(row0 + j) * hidden;
-#pragma unroll
-  for (int g = 0; g < GW; ++g) {
-    if (g_first + g >= groups) continue;
-    const int col = (g_first + g) * 16 + 4 * c;
-#pragma unroll
-    for (int v = 0; v < 4; ++v)
-      if (col + v < hidden) out[col + v].bits = f32_to_bf16(acc[g][v]);
   }
 }
 
@@ -347,25 +390,28 @@ KVF_EXPORT int kvf_moe_grouped(const void* x, int ldx, const void* h, int n, int
                                void* y, float* residual, hipStream_t s) {
   if (n <= 0) return 0;
   const int pairs = n * top;
+  // many rows: tiles of 64 rows (four sub-tiles share every weight fragment); few: tiles of 16
+  const bool many = pairs >= 1024;
+  const int tile_rows = many ? 64 : 16;
   if (E <= 0 || E > PLAN_MAX_EXPERTS || K % 8 != 0 || ff % 32 != 0 || ldx % 8 != 0 || max_tiles > 65535 ||
-      max_tiles < (pairs + TILE_ROWS - 1) / TILE_ROWS + E)
+      max_tiles < (pairs + 15) / 16 + E)
     return static_cast<int>(hipErrorInvalidValue);
   hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, s, sel, pairs, E, where, order, tiles, num_tiles,
-                     max_tiles);
+                     max_tiles, tile_rows);
   const int S = (K + 31) / 32, up_groups = ff / 8, down_groups = (K + 15) / 16;
-  const bool many = pairs >= 1024;
   const int gw = many ? 4 : 2;
-  const dim3 up_grid((up_groups + 4 * gw - 1) / (4 * gw), max_tiles), down_grid((down_groups + 4 * gw - 1) / (4 * gw), max_tiles);
+  const int grid_tiles = many ? (pairs + 63) / 64 + E : max_tiles;
+  const dim3 up_grid((up_groups + 4 * gw - 1) / (4 * gw), grid_tiles), down_grid((down_groups + 4 * gw - 1) / (4 * gw), grid_tiles);
   const bf16_t* xb = static_cast<const bf16_t*>(x);
   if (many) {
-    hipLaunchKernelGGL(moe_up_kernel<4>, up_grid, dim3(256), 0, s, xb, ldx, K, static_cast<const uint4*>(w_gate_up), S,
+    hipLaunchKernelGGL((moe_up_kernel<4, 4>), up_grid, dim3(256), 0, s, xb, ldx, K, static_cast<const uint4*>(w_gate_up), S,
                        order, tiles, num_tiles, top, ff, static_cast<bf16_t*>(act));
-    hipLaunchKernelGGL(moe_down_kernel<4>, down_grid, dim3(256), 0, s, static_cast<const bf16_t*>(act), ff,
+    hipLaunchKernelGGL((moe_down_kernel<4, 4>), down_grid, dim3(256), 0, s, static_cast<const bf16_t*>(act), ff,
                        static_cast<const uint4*>(w_down), E * (ff / 32), tiles, num_tiles, static_cast<bf16_t*>(y), K);
   } else {
-    hipLaunchKernelGGL(moe_up_kernel<2>, up_grid, dim3(256), 0, s, xb, ldx, K, static_cast<const uint4*>(w_gate_up), S,
+    hipLaunchKernelGGL((moe_up_kernel<1, 2>), up_grid, dim3(256), 0, s, xb, ldx, K, static_cast<const uint4*>(w_gate_up), S,
                        order, tiles, num_tiles, top, ff, static_cast<bf16_t*>(act));
-    hipLaunchKernelGGL(moe_down_kernel<2>, down_grid, dim3(256), 0, s, static_cast<const bf16_t*>(act), ff,
+    hipLaunchKernelGGL((moe_down_kernel<1, 2>), down_grid, dim3(256), 0, s, static_cast<const bf16_t*>(act), ff,
                        static_cast<const uint4*>(w_down), E * (ff / 32), tiles, num_tiles, static_cast<bf16_t*>(y), K);
   }
   hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(n), dim3(256), 0, s, residual, static_cast<const bf16_t*>(y),
