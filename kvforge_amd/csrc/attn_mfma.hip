@@ -345,7 +345,8 @@ __device__ __forceinline__ void setup_rows(const bf16_t* q, const MArgs& a, int 
 // ------------------------------------------------------------------------------------ query runs
 // SHARE: the waves stage the fragments of each key block in LDS for each other; otherwise every
 // wave loads all of them itself.
-template <int DT, int RT, bool SHARE, bool BIAS>
+// SINK: the softmax has a sink (a.sinks); a kernel without is the code it was before sinks came
+template <int DT, int RT, bool SHARE, bool BIAS, bool SINK>
 __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
@@ -583,7 +584,9 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
   for (int rt = 0; rt < RT; ++rt) {
     float l = row_sum(l_run[rt]);
     if (!rows.ok[rt]) continue;
-    if (a.sinks && l > 0.f) l += exp2f(fmaf(a.sinks[rows.head[rt]], LOG2E, -m_ref[rt]));
+    if constexpr (SINK) {
+      if (l > 0.f) l += __builtin_amdgcn_exp2f(fmaf(a.sinks[rows.head[rt]], LOG2E, -m_ref[rt]));
+    }
     const float inv = l > 0.f ? 1.f / l : 0.f;
     bf16_t* o = out + static_cast<size_t>(q0 + rows.tok[rt]) * a.o_stride + rows.head[rt] * D + 4 * kg;
     const bf16_t* g = a.gate ? a.gate + static_cast<size_t>(q0 + rows.tok[rt]) * a.gate_stride + rows.head[rt] * D + 4 * kg
@@ -599,7 +602,7 @@ __global__ __launch_bounds__(256) KVF_VGPR_FORM(DT <= 8) void attn_mfma_runs_ker
 // ------------------------------------------------------------------------- few rows, split keys
 // TWO: a wave holds the fragments of two blocks, loading one while it consumes the other.
 // NW: waves of the workgroup; more of them shorten each wave's walk over its cut of the keys.
-template <int DT, bool TWO, int NW, bool BIAS>
+template <int DT, bool TWO, int NW, bool BIAS, bool SINK>
 __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfma_split_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ vt_pages, const int* __restrict__ block_table,
@@ -765,7 +768,9 @@ __global__ __launch_bounds__(NW * KVF_WAVE) KVF_VGPR_FORM(DT <= 6) void attn_mfm
     part_ml[slot * 2] = mm;  // in log2 units
     part_ml[slot * 2 + 1] = ll;
   }
-  if (a.splits == 1 && a.sinks && ll > 0.f) ll += exp2f(fmaf(a.sinks[head], LOG2E, -mm));
+  if constexpr (SINK) {
+    if (a.splits == 1 && ll > 0.f) ll += __builtin_amdgcn_exp2f(fmaf(a.sinks[head], LOG2E, -mm));
+  }
   const float inv = ll > 0.f ? 1.f / ll : 0.f;
   for (int t = wave; t < DT; t += NW) {  // wave w finishes element tiles w, w + NW, ...
     f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -854,13 +859,18 @@ void launch_runs_rt(dim3 grid, hipStream_t s, const void* q, const void* k_pages
   constexpr bool SHARE = runs_share(DT);
   constexpr int N_FRAG = 2 * ((DT + 1) / 2) + DT;
   const size_t lds = SHARE ? static_cast<size_t>(2) * N_FRAG * KVF_WAVE * sizeof(uint4) : 0;
-  if (a.slopes)
-    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, true>), grid, dim3(256), lds, s,
+  if (a.sinks)   // (never with slopes: the exported entry refuses the pair)
+    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, false, true>), grid, dim3(256), lds, s,
+                       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                       static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
+                       static_cast<bf16_t*>(out), a);
+  else if (a.slopes)
+    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, true, false>), grid, dim3(256), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), a);
   else
-    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, false>), grid, dim3(256), lds, s,
+    hipLaunchKernelGGL((attn_mfma_runs_kernel<DT, RT, SHARE, false, false>), grid, dim3(256), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, work, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), a);
@@ -884,13 +894,18 @@ void launch_split_waves(dim3 grid, hipStream_t s, const void* q, const void* k_p
                         const int* block_table, const int* seq_ids, const int* cu_q, const int* ctx_lens,
                         void* out, float* part_acc, float* part_ml, const MArgs& a) {
   const size_t lds = (static_cast<size_t>(NW) * DT * KVF_WAVE * 4 + NW * 16 * 2) * sizeof(float);
-  if (a.slopes)
-    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, true>), grid, dim3(NW * KVF_WAVE), lds, s,
+  if (a.sinks)
+    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, false, true>), grid, dim3(NW * KVF_WAVE), lds, s,
+                       static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
+                       static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
+                       static_cast<bf16_t*>(out), part_acc, part_ml, a);
+  else if (a.slopes)
+    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, true, false>), grid, dim3(NW * KVF_WAVE), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), part_acc, part_ml, a);
   else
-    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, false>), grid, dim3(NW * KVF_WAVE), lds, s,
+    hipLaunchKernelGGL((attn_mfma_split_kernel<DT, (DT <= 8), NW, false, false>), grid, dim3(NW * KVF_WAVE), lds, s,
                        static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k_pages),
                        static_cast<const bf16_t*>(vt_pages), block_table, seq_ids, cu_q, ctx_lens,
                        static_cast<bf16_t*>(out), part_acc, part_ml, a);
@@ -936,7 +951,7 @@ int runs_blocks_per_cu() {
   constexpr int N_FRAG = 2 * ((DT + 1) / 2) + DT;
   const size_t lds = SHARE ? static_cast<size_t>(2) * N_FRAG * KVF_WAVE * sizeof(uint4) : 0;
   int n = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, attn_mfma_runs_kernel<DT, RT, SHARE, false>, 256, lds) !=
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, attn_mfma_runs_kernel<DT, RT, SHARE, false, false>, 256, lds) !=
       hipSuccess)
     return 0;
   return n;
@@ -967,6 +982,7 @@ KVF_EXPORT int kvf_attn_mfma_prefill(const void* q, const void* k_pages, const v
                                      int window, int keep, int n_seqs, float scale, const float* slopes,
                                      const void* gate, int gate_stride, const float* sinks, hipStream_t s) {
   if (num_work <= 0) return 0;
+  if (sinks && slopes) return static_cast<int>(hipErrorInvalidValue);   // no kernel has both
   if (keep < 0 || (gate && (gate_stride % 4 != 0 || gate_stride < H * d || reinterpret_cast<uintptr_t>(gate) % 8 != 0)))
     return static_cast<int>(hipErrorInvalidValue);
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0)
@@ -1000,6 +1016,7 @@ KVF_EXPORT int kvf_attn_mfma_decode(const void* q, const void* k_pages, const vo
                                     int keep, int n_seqs, int splits, float scale, const float* slopes,
                                     const void* gate, int gate_stride, const float* sinks, hipStream_t s) {
   if (num_seqs <= 0) return 0;
+  if (sinks && slopes) return static_cast<int>(hipErrorInvalidValue);
   if (keep < 0 || (gate && (gate_stride % 4 != 0 || gate_stride < H * d || reinterpret_cast<uintptr_t>(gate) % 8 != 0)))
     return static_cast<int>(hipErrorInvalidValue);
   if (!args_ok(H, KV, d, bs, nb, table_stride, scale) || q_stride % 8 != 0 || o_stride % 4 != 0 || splits < 1 ||

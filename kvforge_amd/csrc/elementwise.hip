@@ -507,7 +507,8 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_kernel(
   }
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE, waves = blockDim.x / KVF_WAVE;
   const int heads = a.H + (a.write_kv ? a.KV : 0);
-  for (int hh = wave; hh < heads; hh += waves) {
+  // blockIdx.y names a share of the token's heads (and of its V elements): few tokens still fill the chip
+  for (int hh = blockIdx.y * waves + wave; hh < heads; hh += gridDim.y * waves) {
     const bool is_k = hh >= a.H;
     if (is_k && page < 0) continue;
     T* x = row + hh * a.d;
@@ -539,7 +540,7 @@ __global__ __launch_bounds__(256) void qknorm_rope_kvwrite_kernel(
     }
   }
   if (page < 0) return;
-  for (int t = threadIdx.x; t < a.KV * a.d; t += blockDim.x) {
+  for (int t = blockIdx.y * blockDim.x + threadIdx.x; t < a.KV * a.d; t += gridDim.y * blockDim.x) {
     const int hh = t / a.d, i = t - hh * a.d;
     v_pages[((static_cast<size_t>(page) * a.KV + hh) * a.d + i) * a.block_size + off] =
         row[(a.H + a.KV + hh) * a.d + i];
@@ -554,7 +555,11 @@ static int qknorm_rope_launch(void* qkv, const int* positions, const int* seq_of
   if (n <= 0) return 0;
   if (a.d > 4 * KVF_WAVE || dk > a.d || dk <= 0 || a.rot > dk || a.rot % 2 || !qw || (a.write_kv && !kw))
     return static_cast<int>(hipErrorInvalidValue);
-  hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<T>, dim3(n), dim3(256), 0, s, static_cast<T*>(qkv), positions,
+  // a wave a head where the tokens alone do not fill the chip; four heads a wave for many tokens
+  const int heads = a.H + (a.write_kv ? a.KV : 0);
+  int shares = n >= 1024 ? 1 : (heads + 3) / 4;
+  if (shares > 64) shares = 64;
+  hipLaunchKernelGGL(qknorm_rope_kvwrite_kernel<T>, dim3(n, shares), dim3(256), 0, s, static_cast<T*>(qkv), positions,
                      seq_of_token, cos_t, sin_t, block_table, static_cast<T*>(k_pages),
                      static_cast<T*>(v_pages), qw, kw, dk, eps, a);
   return kvf_last_error();

@@ -210,6 +210,8 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
     return;
   }
   const bool fresh = positions[t0] == 0;
+  const bool vec8 = dk % 8 == 0 && a.row_len % 8 == 0 && a.q_off % 8 == 0 && a.k_off % 8 == 0 &&
+                    reinterpret_cast<uintptr_t>(qkv) % (8 * sizeof(T)) == 0;
   float* st = state + (static_cast<size_t>(slot) * a.H + head) * (static_cast<size_t>(dk) * dv + dk + 1);
   for (int i = tid; i < DKP * CCOLS; i += blockDim.x) {
     const int r = i / CCOLS, c = col0 + i % CCOLS;
@@ -221,16 +223,34 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
   for (int tb = t0; tb < t1; tb += CL) {
     const int cnt = min(CL, t1 - tb);
     __syncthreads();   // the chunk before is done with everything
-    for (int i = tid; i < CL * DKP; i += blockDim.x) {
-      const int t = i / DKP, e = i - t * DKP;
-      float qv = 0.f, kv = 0.f;
-      if (t < cnt && e < dk) {
-        const T* row = qkv + static_cast<size_t>(tb + t) * a.row_len;
-        qv = Elem<T>::load(row + a.q_off + head * dk + e) * a.q_scale;
-        kv = Elem<T>::load(row + a.k_off + head * dk + e);
+    if (vec8) {
+      // eight elements a load: the heads' rows start on 16 bytes (32 for fp32) and dk is a multiple of 8
+      for (int i = tid; i < CL * (DKP / 8); i += blockDim.x) {
+        const int t = i / (DKP / 8), e = 8 * (i - t * (DKP / 8));
+        float qv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, kv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (t < cnt && e < dk) {
+          const T* row = qkv + static_cast<size_t>(tb + t) * a.row_len;
+          load8(row + a.q_off + head * dk + e, qv);
+          load8(row + a.k_off + head * dk + e, kv);
+        }
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+          Qs[t * QLD + e + x] = qv[x] * a.q_scale;
+          Ks[t * QLD + e + x] = kv[x];
+        }
       }
-      Qs[t * QLD + e] = qv;
-      Ks[t * QLD + e] = kv;
+    } else {
+      for (int i = tid; i < CL * DKP; i += blockDim.x) {
+        const int t = i / DKP, e = i - t * DKP;
+        float qv = 0.f, kv = 0.f;
+        if (t < cnt && e < dk) {
+          const T* row = qkv + static_cast<size_t>(tb + t) * a.row_len;
+          qv = Elem<T>::load(row + a.q_off + head * dk + e) * a.q_scale;
+          kv = Elem<T>::load(row + a.k_off + head * dk + e);
+        }
+        Qs[t * QLD + e] = qv;
+        Ks[t * QLD + e] = kv;
+      }
     }
     for (int i = tid; i < CL * CCOLS; i += blockDim.x) {
       const int t = i / CCOLS, c = col0 + i % CCOLS;

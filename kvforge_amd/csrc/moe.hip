@@ -328,13 +328,29 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x,
   const int n = blockIdx.x;
   float* xr = x + static_cast<size_t>(n) * hidden;
   const T* hr = h + static_cast<size_t>(n) * hidden;
+  // a token's choices once, then the elements with nothing but independent loads
+  float w[MAX_TOP];
+  const bf16_t* src[MAX_TOP];
+  bool own[MAX_TOP];
+#pragma unroll
+  for (int k = 0; k < MAX_TOP; ++k) {
+    w[k] = 0.f;
+    src[k] = nullptr;
+    own[k] = false;
+    if (k < top) {
+      const int p = n * top + k, e = sel[p];
+      w[k] = wgt[p];
+      own[k] = e >= E;
+      if (e >= 0 && e < E) src[k] = y + static_cast<size_t>(where[p]) * hidden;
+    }
+  }
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float sum = 0.f;
-    for (int k = 0; k < top; ++k) {
-      const int p = n * top + k, e = sel[p];
-      const float w = wgt[p];
-      if (e >= E) sum = fmaf(w, Elem<T>::load(hr + i), sum);
-      else if (e >= 0) sum = fmaf(w, bf16_to_f32(y[static_cast<size_t>(where[p]) * hidden + i].bits), sum);
+#pragma unroll
+    for (int k = 0; k < MAX_TOP; ++k) {
+      if (k >= top) break;
+      if (own[k]) sum = fmaf(w[k], Elem<T>::load(hr + i), sum);
+      else if (src[k]) sum = fmaf(w[k], bf16_to_f32(src[k][i].bits), sum);
     }
     xr[i] += sum;
   }
@@ -399,7 +415,7 @@ KVF_EXPORT int kvf_moe_grouped(const void* x, int ldx, const void* h, int n, int
   hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(1024), 0, s, sel, pairs, E, where, order, tiles, num_tiles,
                      max_tiles, tile_rows);
   const int S = (K + 31) / 32, up_groups = ff / 8, down_groups = (K + 15) / 16;
-  const int gw = many ? 4 : 2;
+  const int gw = many ? 4 : 1;
   const int grid_tiles = many ? (pairs + 63) / 64 + E : max_tiles;
   const dim3 up_grid((up_groups + 4 * gw - 1) / (4 * gw), grid_tiles), down_grid((down_groups + 4 * gw - 1) / (4 * gw), grid_tiles);
   const bf16_t* xb = static_cast<const bf16_t*>(x);
@@ -409,9 +425,9 @@ KVF_EXPORT int kvf_moe_grouped(const void* x, int ldx, const void* h, int n, int
     hipLaunchKernelGGL((moe_down_kernel<4, 4>), down_grid, dim3(256), 0, s, static_cast<const bf16_t*>(act), ff,
                        static_cast<const uint4*>(w_down), E * (ff / 32), tiles, num_tiles, static_cast<bf16_t*>(y), K);
   } else {
-    hipLaunchKernelGGL((moe_up_kernel<1, 2>), up_grid, dim3(256), 0, s, xb, ldx, K, static_cast<const uint4*>(w_gate_up), S,
+    hipLaunchKernelGGL((moe_up_kernel<1, 1>), up_grid, dim3(256), 0, s, xb, ldx, K, static_cast<const uint4*>(w_gate_up), S,
                        order, tiles, num_tiles, top, ff, static_cast<bf16_t*>(act));
-    hipLaunchKernelGGL((moe_down_kernel<1, 2>), down_grid, dim3(256), 0, s, static_cast<const bf16_t*>(act), ff,
+    hipLaunchKernelGGL((moe_down_kernel<1, 1>), down_grid, dim3(256), 0, s, static_cast<const bf16_t*>(act), ff,
                        static_cast<const uint4*>(w_down), E * (ff / 32), tiles, num_tiles, static_cast<bf16_t*>(y), K);
   }
   hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, dim3(n), dim3(256), 0, s, residual, static_cast<const bf16_t*>(y),

@@ -937,6 +937,11 @@ def _sinks_ptr(sinks, H: int, like: torch.Tensor):
     return sinks.data_ptr()
 
 
+def _no_sinks_with_slopes(sinks, slopes, on_matrix_cores: bool) -> None:
+    if sinks is not None and slopes is not None and on_matrix_cores:
+        raise KernelError("attention: the matrix-core kernels take sinks or slopes, not both")
+
+
 def _keep_first(window: int, keep_first: int) -> int:
     """Keys kept visible behind a window; without a window every key is visible anyway."""
     keep = int(keep_first)
@@ -1016,6 +1021,7 @@ def attn_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
     nb, _, bs, _ = k_pages.shape
     if rows_per_item is None:
         rows_per_item = prefill_rows_per_item(q.dtype, d, bs)
+    _no_sinks_with_slopes(sinks, slopes, attention_on_matrix_cores(q.dtype, bs))
     if attention_on_matrix_cores(q.dtype, bs):
         f = _fn("attn_mfma", "kvf_attn_mfma_prefill",
                 [c_void_p] * 7 + [c_int, c_int] + [c_void_p] + [c_int] * 11 + [c_float, c_void_p, c_void_p, c_int, c_void_p, c_void_p])
@@ -1083,6 +1089,7 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
         _check(pm, "workspace[1]", F32)
         if pa.numel() < num_seqs * H * splits * d or pm.numel() < num_seqs * H * splits * 2:
             raise KernelError("attn_decode: workspace too small")
+    _no_sinks_with_slopes(sinks, slopes, attention_on_matrix_cores(q.dtype, bs))
     if not attention_on_matrix_cores(q.dtype, bs):
         if gate is not None:
             raise KernelError("attn_decode: the 32-bit kernel takes no gate; gate its rows afterwards")
