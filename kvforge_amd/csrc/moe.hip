@@ -319,6 +319,11 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const bf16_t* __restrict_
 
 // x[n, :] += sum over the token's choices, in their order, of weight * (the expert's row of y, or
 // the token's own input h for a choice that names no expert): fp32 sums into the fp32 stream.
+// A thread takes eight neighbouring elements (hidden is a multiple of 8 here): per choice one
+// 16-byte load, the choice itself being the same for the whole workgroup.
+__device__ __forceinline__ void load8_any(const bf16_t* p, float (&v)[8]) { load8(p, v); }
+__device__ __forceinline__ void load8_any(const float* p, float (&v)[8]) { load8(p, v); }
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x, const bf16_t* __restrict__ y,
                                                           const T* __restrict__ h, const int* __restrict__ sel,
@@ -328,31 +333,23 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ x,
   const int n = blockIdx.x;
   float* xr = x + static_cast<size_t>(n) * hidden;
   const T* hr = h + static_cast<size_t>(n) * hidden;
-  // a token's choices once, then the elements with nothing but independent loads
-  float w[MAX_TOP];
-  const bf16_t* src[MAX_TOP];
-  bool own[MAX_TOP];
-#pragma unroll
-  for (int k = 0; k < MAX_TOP; ++k) {
-    w[k] = 0.f;
-    src[k] = nullptr;
-    own[k] = false;
-    if (k < top) {
+  for (int i = 8 * threadIdx.x; i < hidden; i += 8 * blockDim.x) {
+    float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < top; ++k) {
       const int p = n * top + k, e = sel[p];
-      w[k] = wgt[p];
-      own[k] = e >= E;
-      if (e >= 0 && e < E) src[k] = y + static_cast<size_t>(where[p]) * hidden;
-    }
-  }
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    float sum = 0.f;
+      const float w = wgt[p];
+      float v[8];
+      if (e >= E) load8_any(hr + i, v);
+      else if (e >= 0) load8(y + static_cast<size_t>(where[p]) * hidden + i, v);
+      else continue;
 #pragma unroll
-    for (int k = 0; k < MAX_TOP; ++k) {
-      if (k >= top) break;
-      if (own[k]) sum = fmaf(w[k], Elem<T>::load(hr + i), sum);
-      else if (src[k]) sum = fmaf(w[k], bf16_to_f32(src[k][i].bits), sum);
+      for (int u = 0; u < 8; ++u) sum[u] = fmaf(w, v[u], sum[u]);
     }
-    xr[i] += sum;
+    float4 a = *reinterpret_cast<const float4*>(xr + i), b = *reinterpret_cast<const float4*>(xr + i + 4);
+    a.x += sum[0]; a.y += sum[1]; a.z += sum[2]; a.w += sum[3];
+    b.x += sum[4]; b.y += sum[5]; b.z += sum[6]; b.w += sum[7];
+    *reinterpret_cast<float4*>(xr + i) = a;
+    *reinterpret_cast<float4*>(xr + i + 4) = b;
   }
 }
 }  // namespace
