@@ -36,7 +36,7 @@ __global__ __launch_bounds__(ROWS > KVF_WAVE ? 2 * KVF_WAVE : KVF_WAVE) void mls
                                   const float* __restrict__ bias_if, const int* __restrict__ cu_q,
                                   const int* __restrict__ positions, const int* __restrict__ slot_ids,
                                   float* __restrict__ state, float* __restrict__ out, ScanArgs a) {
-  extern __shared__ float lds[];
+  extern __shared__ __align__(16) float lds[];
   const int seq = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * COLS;
   const int lane = threadIdx.x % KVF_WAVE, wave = threadIdx.x / KVF_WAVE, RG = blockDim.x / KVF_WAVE;
   const int slot = slot_ids[seq];
@@ -163,8 +163,11 @@ __global__ __launch_bounds__(ROWS > KVF_WAVE ? 2 * KVF_WAVE : KVF_WAVE) void mls
 //   A = (Q K^T) * D;   O = A V + diag(g) Q S;   n_t . q_t = rowsum(A)_t + g_t q_t . n
 //   S' = g_L S + K^T diag(D[L]) V;   n' = g_L n + K^T D[L];   m_c' = m_L        (L: the last token)
 // which is the recurrence written out over the chunk.  A workgroup of four waves takes 32 columns
-// of S for one (sequence, head); Q, K (fp32, rows padded to an odd stride), the V columns, A and
-// the S columns live in LDS.
+// of S for one (sequence, head); Q, K, A (fp32, token-major) and V, S (column-major: Vt[c][token],
+// St[c][k]) live in LDS with row strides of 4 mod 32 floats.  The four lane groups of the
+// instruction stand for four *neighbouring* k each (group g takes k = k0 + 4 g + e in
+// instruction e of four), so that a lane's operands for four instructions are 16 consecutive
+// bytes of a row: one LDS read for four matrix instructions, spread evenly over the banks.
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int CCOLS = 32;
 
@@ -176,18 +179,18 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
                                                           const int* __restrict__ slot_ids,
                                                           float* __restrict__ state, float* __restrict__ out,
                                                           ScanArgs a) {
-  extern __shared__ float lds[];
-  constexpr int QLD = DKP + 1, ALD = CL + 1;
+  extern __shared__ __align__(16) float lds[];
+  constexpr int QLD = DKP + 4, ALD = CL + 4, VLD = CL + 4, SLD = DKP + 4;
   // the running sum of the log forget gates is kept in 64 bits: its differences b_t - b_s are
   // what the weights are made of, and a sum that has passed a nearly closed gate is hundreds
   // of times larger than the differences that matter behind it
   double* bc = reinterpret_cast<double*>(lds);   // [CL] log forget gates, then their running sum
   float* Qs = lds + 2 * CL;              // [CL][QLD], q times its scale
   float* Ks = Qs + CL * QLD;             // [CL][QLD]
-  float* Vs = Ks + CL * QLD;             // [CL][CCOLS]
-  float* As = Vs + CL * CCOLS;           // [CL][ALD]
-  float* Ss = As + CL * ALD;             // [DKP][CCOLS]
-  float* ns = Ss + DKP * CCOLS;          // [DKP]
+  float* Vt = Ks + CL * QLD;             // [CCOLS][VLD]: the block's columns of v, a column's tokens side by side
+  float* As = Vt + CCOLS * VLD;          // [CL][ALD]
+  float* St = As + CL * ALD;             // [CCOLS][SLD]: the block's columns of S, a column's rows side by side
+  float* ns = St + CCOLS * SLD;          // [DKP]
   float* li = ns + DKP;                  // [CL] log input gates
   float* mt = li + CL;                   // [CL] running maximum after each token
   float* gt = mt + CL;                   // [CL] weight of the chunk's first state for token t
@@ -214,8 +217,8 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
                     reinterpret_cast<uintptr_t>(qkv) % (8 * sizeof(T)) == 0;
   float* st = state + (static_cast<size_t>(slot) * a.H + head) * (static_cast<size_t>(dk) * dv + dk + 1);
   for (int i = tid; i < DKP * CCOLS; i += blockDim.x) {
-    const int r = i / CCOLS, c = col0 + i % CCOLS;
-    Ss[i] = (!fresh && r < dk && c < dv) ? st[static_cast<size_t>(r) * dv + c] : 0.f;
+    const int r = i / CCOLS, cl = i % CCOLS, c = col0 + cl;
+    St[cl * SLD + r] = (!fresh && r < dk && c < dv) ? st[static_cast<size_t>(r) * dv + c] : 0.f;
   }
   for (int r = tid; r < DKP; r += blockDim.x) ns[r] = (!fresh && r < dk) ? st[static_cast<size_t>(dk) * dv + r] : 0.f;
   if (tid == 0) m_c = fresh ? 0.f : st[static_cast<size_t>(dk) * dv + dk];
@@ -253,10 +256,10 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
       }
     }
     for (int i = tid; i < CL * CCOLS; i += blockDim.x) {
-      const int t = i / CCOLS, c = col0 + i % CCOLS;
-      Vs[i] = (t < cnt && c < dv)
-                  ? Elem<T>::load(qkv + static_cast<size_t>(tb + t) * a.row_len + a.v_off + head * dv + c)
-                  : 0.f;
+      const int t = i / CCOLS, cl = i % CCOLS, c = col0 + cl;
+      Vt[cl * VLD + t] = (t < cnt && c < dv)
+                             ? Elem<T>::load(qkv + static_cast<size_t>(tb + t) * a.row_len + a.v_off + head * dv + c)
+                             : 0.f;
     }
     if (wave == 0) {
       // a lane per token: the gates, the running sum of the log forget gates (64-bit) and the
@@ -302,10 +305,14 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
       const int rt = tile / RT, ct = tile - rt * RT;
       f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
       if (ct <= rt) {
-        const float* qa = Qs + (16 * rt + l16) * QLD + lq;
-        const float* kb = Ks + (16 * ct + l16) * QLD + lq;
-#pragma unroll 8
-        for (int k0 = 0; k0 < DKP; k0 += 4) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[k0], kb[k0], acc, 0, 0, 0);
+        const float* qa = Qs + (16 * rt + l16) * QLD + 4 * lq;
+        const float* kb = Ks + (16 * ct + l16) * QLD + 4 * lq;
+#pragma unroll 4
+        for (int k0 = 0; k0 < DKP; k0 += 16) {
+          const f32x4 a4 = *reinterpret_cast<const f32x4*>(qa + k0), b4 = *reinterpret_cast<const f32x4*>(kb + k0);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[e], b4[e], acc, 0, 0, 0);
+        }
       }
       const int s = 16 * ct + l16;
 #pragma unroll
@@ -338,16 +345,22 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
     for (int tile = wave; tile < RT * (CCOLS / 16); tile += 4) {
       const int rt = tile / (CCOLS / 16), ct = tile - rt * (CCOLS / 16);
       f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
-      const float* aa = As + (16 * rt + l16) * ALD + lq;
-      const float* vb = Vs + lq * CCOLS + 16 * ct + l16;
-      for (int k0 = 0; k0 < 16 * (rt + 1); k0 += 4)
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(aa[k0], vb[k0 * CCOLS], acc, 0, 0, 0);
+      const float* aa = As + (16 * rt + l16) * ALD + 4 * lq;
+      const float* vb = Vt + (16 * ct + l16) * VLD + 4 * lq;
+      for (int k0 = 0; k0 < 16 * (rt + 1); k0 += 16) {
+        const f32x4 a4 = *reinterpret_cast<const f32x4*>(aa + k0), b4 = *reinterpret_cast<const f32x4*>(vb + k0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[e], b4[e], acc, 0, 0, 0);
+      }
       const float g = gt[16 * rt + l16];
-      const float* qa = Qs + (16 * rt + l16) * QLD + lq;
-      const float* sb = Ss + lq * CCOLS + 16 * ct + l16;
-#pragma unroll 8
-      for (int k0 = 0; k0 < DKP; k0 += 4)
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[k0] * g, sb[k0 * CCOLS], acc, 0, 0, 0);
+      const float* qa = Qs + (16 * rt + l16) * QLD + 4 * lq;
+      const float* sb = St + (16 * ct + l16) * SLD + 4 * lq;
+#pragma unroll 4
+      for (int k0 = 0; k0 < DKP; k0 += 16) {
+        const f32x4 a4 = *reinterpret_cast<const f32x4*>(qa + k0) * g, b4 = *reinterpret_cast<const f32x4*>(sb + k0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[e], b4[e], acc, 0, 0, 0);
+      }
       const int c = col0 + 16 * ct + l16;
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
@@ -360,16 +373,19 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
     const float g_last = gt[last];
     for (int tile = wave; tile < (DKP / 16) * (CCOLS / 16); tile += 4) {
       const int kt = tile / (CCOLS / 16), ct = tile - kt * (CCOLS / 16);
-      f32x4 acc;
+      // the lane's four rows of S are neighbours in St: one read, one write
+      f32x4* mine = reinterpret_cast<f32x4*>(St + (16 * ct + l16) * SLD + 16 * kt + 4 * lq);
+      f32x4 acc = *mine * g_last;
+      const float* ka = Ks + (4 * lq) * QLD + 16 * kt + l16;
+      const float* vb = Vt + (16 * ct + l16) * VLD + 4 * lq;
+#pragma unroll 2
+      for (int k0 = 0; k0 < CL; k0 += 16) {
+        const f32x4 b4 = *reinterpret_cast<const f32x4*>(vb + k0) * *reinterpret_cast<const f32x4*>(wl + k0 + 4 * lq);
 #pragma unroll
-      for (int v = 0; v < 4; ++v) acc[v] = g_last * Ss[(16 * kt + 4 * lq + v) * CCOLS + 16 * ct + l16];
-      const float* ka = Ks + lq * QLD + 16 * kt + l16;
-      const float* vb = Vs + lq * CCOLS + 16 * ct + l16;
-#pragma unroll 8
-      for (int k0 = 0; k0 < CL; k0 += 4)
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[k0 * QLD], vb[k0 * CCOLS] * wl[k0 + lq], acc, 0, 0, 0);
-#pragma unroll
-      for (int v = 0; v < 4; ++v) Ss[(16 * kt + 4 * lq + v) * CCOLS + 16 * ct + l16] = acc[v];
+        for (int e = 0; e < 4; ++e)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[(k0 + e) * QLD], b4[e], acc, 0, 0, 0);
+      }
+      *mine = acc;
     }
     for (int k = tid; k < DKP; k += blockDim.x) {
       float nk = g_last * ns[k];
@@ -380,8 +396,8 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
   }
   __syncthreads();
   for (int i = tid; i < DKP * CCOLS; i += blockDim.x) {
-    const int r = i / CCOLS, c = col0 + i % CCOLS;
-    if (r < dk && c < dv) st[static_cast<size_t>(r) * dv + c] = Ss[i];
+    const int r = i / CCOLS, cl = i % CCOLS, c = col0 + cl;
+    if (r < dk && c < dv) st[static_cast<size_t>(r) * dv + c] = St[cl * SLD + r];
   }
   if (blockIdx.x == 0) {
     for (int r = tid; r < dk; r += blockDim.x) st[static_cast<size_t>(dk) * dv + r] = ns[r];
@@ -390,7 +406,8 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
 }
 
 template <int DKP, int CL> constexpr size_t chunk_lds() {
-  return sizeof(float) * (2 * CL * (DKP + 1) + CL * CCOLS + CL * (CL + 1) + DKP * CCOLS + DKP + 7 * CL + 256);
+  return sizeof(float) * (2 * CL + 2 * CL * (DKP + 4) + CCOLS * (CL + 4) + CL * (CL + 4) + CCOLS * (DKP + 4) + DKP +
+                          5 * CL + 256);
 }
 
 template <typename T, int DKP, int CL>
