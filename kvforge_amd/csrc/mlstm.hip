@@ -20,6 +20,7 @@ struct ScanArgs {
   float cap, q_scale;
   int gate_stride;          // numbers from one token's gate row to the next (at least 2 H)
   int chunk_from;           // runs of at least so many tokens are the chunk kernel's, shorter ones the scan kernel's
+  int multi_from;           // and runs of at least so many are taken by the kernels that work on all chunks at once
 };
 
 __device__ __forceinline__ float capped(float z, float cap) { return cap * tanhf(z / cap); }
@@ -203,7 +204,7 @@ __global__ __launch_bounds__(256) void mlstm_chunk_kernel(const T* __restrict__ 
   const int l16 = lane % 16, lq = lane / 16;
   const int slot = slot_ids[seq];
   const int t0 = cu_q[seq], t1 = cu_q[seq + 1];
-  if (t1 - t0 < a.chunk_from) return;    // short runs belong to the scan kernel
+  if (t1 - t0 < a.chunk_from || t1 - t0 >= a.multi_from) return;    // short runs belong to the scan kernel, the longest to the passes
   const int dk = a.dk, dv = a.dv;
   if (slot < 0 || slot >= a.n_slots) {
     for (int i = tid; i < (t1 - t0) * CCOLS; i += blockDim.x) {
@@ -439,6 +440,371 @@ int chunk_launch(const void* qkv, const float* zif, const float* bias_if, const 
 #undef GO
 }
 
+// ---------------------------------------------------------------------------------------------
+// The longest runs: all chunks of all sequences at once, in four passes (same formulas as above).
+//   gates:  per (sequence, head) one wave walks the chunks: li, b (64-bit), m per token; per chunk
+//           the maximum it starts from (m_c) and the weight of its first state in its last (g_L)
+//   local:  per chunk, U = K^T diag(D[L]) V and u = K^T D[L]: what the chunk adds to the state
+//   carry:  per element of S (and n), over the sequence's chunks in order: the chunk's slot in the
+//           workspace gets the state *before* the chunk, the state becomes g_L S + U
+//   output: per chunk, A = (Q K^T) * D, O = A V + diag(g) Q S_c, the denominator, to memory
+// `chunks` rows: (sequence, first token, tokens, -); `runs` rows: (sequence, first chunk, chunks).
+struct MultiArgs {
+  const int* chunks;
+  const int* runs;
+  float* li;      // [tokens, H]
+  float* mt;      // [tokens, H]
+  double* bc;     // [tokens, H]
+  float* mc;      // [chunks, H] the maximum before the chunk
+  float* gl;      // [chunks, H] exp(b_L + m_c - m_L)
+  float* W;       // [chunks, H, dk, dv]: U after `local`, the state before the chunk after `carry`
+  float* un;      // [chunks, H, dk] likewise for n
+};
+
+template <int CL>
+__global__ __launch_bounds__(KVF_WAVE) void mlstm_gates_kernel(const float* __restrict__ zif,
+                                                               const float* __restrict__ bias_if,
+                                                               const int* __restrict__ cu_q,
+                                                               const int* __restrict__ positions,
+                                                               const int* __restrict__ slot_ids,
+                                                               float* __restrict__ state, ScanArgs a, MultiArgs w) {
+  const int head = blockIdx.x, lane = threadIdx.x;
+  const int seq = w.runs[3 * blockIdx.y], c0 = w.runs[3 * blockIdx.y + 1], nc = w.runs[3 * blockIdx.y + 2];
+  const int slot = slot_ids[seq];
+  if (slot < 0 || slot >= a.n_slots) return;
+  const int t0 = cu_q[seq], t1 = cu_q[seq + 1];
+  float* st = state + (static_cast<size_t>(slot) * a.H + head) * (static_cast<size_t>(a.dk) * a.dv + a.dk + 1);
+  float m_c = positions[t0] == 0 ? 0.f : st[static_cast<size_t>(a.dk) * a.dv + a.dk];
+  for (int j = 0; j < nc; ++j) {
+    const int tb = t0 + j * CL, cnt = min(CL, t1 - tb), t = lane;
+    float i_gate = 0.f, f_gate = 0.f;
+    if (t < cnt) {
+      const float* z = zif + static_cast<size_t>(tb + t) * a.gate_stride;
+      i_gate = capped(z[head] + bias_if[head], a.cap);
+      f_gate = log_sigmoid(capped(z[a.H + head] + bias_if[a.H + head], a.cap));
+    }
+    double b = static_cast<double>(f_gate);
+#pragma unroll
+    for (int o = 1; o < KVF_WAVE; o <<= 1) {
+      const double up = __shfl_up(b, o, KVF_WAVE);
+      if (lane >= o) b += up;
+    }
+    double u = t < cnt ? static_cast<double>(i_gate) - b : -1e300;
+#pragma unroll
+    for (int o = 1; o < KVF_WAVE; o <<= 1) {
+      const double up = __shfl_up(u, o, KVF_WAVE);
+      if (lane >= o) u = fmax(u, up);
+    }
+    const float m = static_cast<float>(b + fmax(static_cast<double>(m_c), u));
+    const double b_last = __shfl(b, cnt - 1, KVF_WAVE);
+    const float m_last = __shfl(m, cnt - 1, KVF_WAVE);
+    if (t < cnt) {
+      const size_t at = static_cast<size_t>(tb + t) * a.H + head;
+      w.li[at] = i_gate;
+      w.bc[at] = b;
+      w.mt[at] = m;
+    }
+    if (lane == 0) {
+      w.mc[static_cast<size_t>(c0 + j) * a.H + head] = m_c;
+      w.gl[static_cast<size_t>(c0 + j) * a.H + head] =
+          expf(static_cast<float>(b_last + static_cast<double>(m_c) - static_cast<double>(m_last)));
+    }
+    m_c = m_last;
+  }
+  if (lane == 0) st[static_cast<size_t>(a.dk) * a.dv + a.dk] = m_c;
+}
+
+// K (token-major) and the block's columns of V (column-major) of one chunk into LDS, as the
+// chunk kernel keeps them; rows past the chunk's tokens and elements past dk, dv are zero.
+template <typename T, int DKP, int CL>
+__device__ __forceinline__ void stage_kv(const T* __restrict__ qkv, const ScanArgs& a, int head, int tb, int cnt,
+                                         int col0, float* Qs, float* Ks, float* Vt, bool vec8) {
+  constexpr int QLD = DKP + 4, VLD = CL + 4;
+  const int tid = threadIdx.x, dk = a.dk, dv = a.dv;
+  if (vec8) {
+    for (int i = tid; i < CL * (DKP / 8); i += blockDim.x) {
+      const int t = i / (DKP / 8), e = 8 * (i - t * (DKP / 8));
+      float qv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, kv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (t < cnt && e < dk) {
+        const T* row = qkv + static_cast<size_t>(tb + t) * a.row_len;
+        if (Qs) load8(row + a.q_off + head * dk + e, qv);
+        load8(row + a.k_off + head * dk + e, kv);
+      }
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        if (Qs) Qs[t * QLD + e + x] = qv[x] * a.q_scale;
+        Ks[t * QLD + e + x] = kv[x];
+      }
+    }
+  } else {
+    for (int i = tid; i < CL * DKP; i += blockDim.x) {
+      const int t = i / DKP, e = i - t * DKP;
+      float qv = 0.f, kv = 0.f;
+      if (t < cnt && e < dk) {
+        const T* row = qkv + static_cast<size_t>(tb + t) * a.row_len;
+        if (Qs) qv = Elem<T>::load(row + a.q_off + head * dk + e) * a.q_scale;
+        kv = Elem<T>::load(row + a.k_off + head * dk + e);
+      }
+      if (Qs) Qs[t * QLD + e] = qv;
+      Ks[t * QLD + e] = kv;
+    }
+  }
+  for (int i = tid; i < CL * CCOLS; i += blockDim.x) {
+    const int t = i / CCOLS, cl = i % CCOLS, c = col0 + cl;
+    Vt[cl * VLD + t] = (t < cnt && c < dv)
+                           ? Elem<T>::load(qkv + static_cast<size_t>(tb + t) * a.row_len + a.v_off + head * dv + c)
+                           : 0.f;
+  }
+}
+
+template <typename T, int DKP, int CL>
+__global__ __launch_bounds__(256) void mlstm_local_kernel(const T* __restrict__ qkv, const int* __restrict__ slot_ids,
+                                                          ScanArgs a, MultiArgs w) {
+  extern __shared__ __align__(16) float lds[];
+  constexpr int QLD = DKP + 4, VLD = CL + 4;
+  float* Ks = lds;                 // [CL][QLD]
+  float* Vt = Ks + CL * QLD;       // [CCOLS][VLD]
+  float* wl = Vt + CCOLS * VLD;    // [CL]
+  const int chunk = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * CCOLS;
+  const int seq = w.chunks[4 * chunk], tb = w.chunks[4 * chunk + 1], cnt = w.chunks[4 * chunk + 2];
+  const int slot = slot_ids[seq];
+  if (slot < 0 || slot >= a.n_slots) return;
+  const int tid = threadIdx.x, lane = tid % KVF_WAVE, wave = tid / KVF_WAVE, l16 = lane % 16, lq = lane / 16;
+  const int dk = a.dk, dv = a.dv;
+  const bool vec8 = dk % 8 == 0 && a.row_len % 8 == 0 && a.k_off % 8 == 0 &&
+                    reinterpret_cast<uintptr_t>(qkv) % (8 * sizeof(T)) == 0;
+  stage_kv<T, DKP, CL>(qkv, a, head, tb, cnt, col0, nullptr, Ks, Vt, vec8);
+  if (tid < CL) {
+    float v = 0.f;
+    if (tid < cnt) {
+      const size_t at = static_cast<size_t>(tb + tid) * a.H + head, last = static_cast<size_t>(tb + cnt - 1) * a.H + head;
+      v = expf(static_cast<float>(w.bc[last] - w.bc[at]) + w.li[at] - w.mt[last]);
+    }
+    wl[tid] = v;
+  }
+  __syncthreads();
+  float* U = w.W + (static_cast<size_t>(chunk) * a.H + head) * dk * dv;
+  for (int tile = wave; tile < (DKP / 16) * (CCOLS / 16); tile += 4) {
+    const int kt = tile / (CCOLS / 16), ct = tile - kt * (CCOLS / 16);
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    const float* ka = Ks + (4 * lq) * QLD + 16 * kt + l16;
+    const float* vb = Vt + (16 * ct + l16) * VLD + 4 * lq;
+#pragma unroll 2
+    for (int k0 = 0; k0 < CL; k0 += 16) {
+      const f32x4 b4 = *reinterpret_cast<const f32x4*>(vb + k0) * *reinterpret_cast<const f32x4*>(wl + k0 + 4 * lq);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[(k0 + e) * QLD], b4[e], acc, 0, 0, 0);
+    }
+    const int c = col0 + 16 * ct + l16;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int k = 16 * kt + 4 * lq + v;
+      if (k < dk && c < dv) U[static_cast<size_t>(k) * dv + c] = acc[v];
+    }
+  }
+  if (blockIdx.x == 0) {
+    float* u = w.un + (static_cast<size_t>(chunk) * a.H + head) * dk;
+    for (int k = tid; k < dk; k += blockDim.x) {
+      float nk = 0.f;
+      for (int s2 = 0; s2 < cnt; ++s2) nk = fmaf(wl[s2], Ks[s2 * QLD + k], nk);
+      u[k] = nk;
+    }
+  }
+}
+
+// One thread per element of a head's S and n, over the run's chunks in order.
+__global__ __launch_bounds__(256) void mlstm_carry_kernel(const int* __restrict__ cu_q, const int* __restrict__ positions,
+                                                          const int* __restrict__ slot_ids, float* __restrict__ state,
+                                                          ScanArgs a, MultiArgs w) {
+  const int head = blockIdx.y;
+  const int seq = w.runs[3 * blockIdx.z], c0 = w.runs[3 * blockIdx.z + 1], nc = w.runs[3 * blockIdx.z + 2];
+  const int slot = slot_ids[seq];
+  if (slot < 0 || slot >= a.n_slots) return;
+  const size_t mat = static_cast<size_t>(a.dk) * a.dv;
+  const size_t e = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (e >= mat + a.dk) return;
+  float* st = state + (static_cast<size_t>(slot) * a.H + head) * (mat + a.dk + 1);
+  float S = positions[cu_q[seq]] == 0 ? 0.f : st[e];
+  for (int j = 0; j < nc; ++j) {
+    const size_t ch = static_cast<size_t>(c0 + j) * a.H + head;
+    float* slot_of = e < mat ? w.W + ch * mat + e : w.un + ch * a.dk + (e - mat);
+    const float add = *slot_of;
+    *slot_of = S;
+    S = fmaf(w.gl[ch], S, add);
+  }
+  st[e] = S;
+}
+
+template <typename T, int DKP, int CL>
+__global__ __launch_bounds__(256) void mlstm_output_kernel(const T* __restrict__ qkv, const int* __restrict__ slot_ids,
+                                                           float* __restrict__ out, ScanArgs a, MultiArgs w) {
+  extern __shared__ __align__(16) float lds[];
+  constexpr int QLD = DKP + 4, ALD = CL + 4, VLD = CL + 4, SLD = DKP + 4;
+  double* bc = reinterpret_cast<double*>(lds);   // [CL]
+  float* Qs = lds + 2 * CL;
+  float* Ks = Qs + CL * QLD;
+  float* Vt = Ks + CL * QLD;
+  float* As = Vt + CCOLS * VLD;
+  float* St = As + CL * ALD;
+  float* ns = St + CCOLS * SLD;
+  float* li = ns + DKP;
+  float* mt = li + CL;
+  float* gt = mt + CL;
+  float* den = gt + CL;
+  float* part = den + CL;   // [256 / CL][CL]
+  const int chunk = blockIdx.z, head = blockIdx.y, col0 = blockIdx.x * CCOLS;
+  const int seq = w.chunks[4 * chunk], tb = w.chunks[4 * chunk + 1], cnt = w.chunks[4 * chunk + 2];
+  const int tid = threadIdx.x, lane = tid % KVF_WAVE, wave = tid / KVF_WAVE, l16 = lane % 16, lq = lane / 16;
+  const int dk = a.dk, dv = a.dv;
+  const int slot = slot_ids[seq];
+  if (slot < 0 || slot >= a.n_slots) {
+    for (int i = tid; i < cnt * CCOLS; i += blockDim.x) {
+      const int t = i / CCOLS, c = col0 + i % CCOLS;
+      if (c < dv) out[static_cast<size_t>(tb + t) * a.H * dv + head * dv + c] = 0.f;
+    }
+    return;
+  }
+  const bool vec8 = dk % 8 == 0 && a.row_len % 8 == 0 && a.q_off % 8 == 0 && a.k_off % 8 == 0 &&
+                    reinterpret_cast<uintptr_t>(qkv) % (8 * sizeof(T)) == 0;
+  stage_kv<T, DKP, CL>(qkv, a, head, tb, cnt, col0, Qs, Ks, Vt, vec8);
+  const size_t ch = static_cast<size_t>(chunk) * a.H + head;
+  const float* Sc = w.W + ch * dk * dv;
+  for (int i = tid; i < DKP * CCOLS; i += blockDim.x) {
+    const int r = i / CCOLS, cl = i % CCOLS, c = col0 + cl;
+    St[cl * SLD + r] = (r < dk && c < dv) ? Sc[static_cast<size_t>(r) * dv + c] : 0.f;
+  }
+  for (int r = tid; r < DKP; r += blockDim.x) ns[r] = r < dk ? w.un[ch * dk + r] : 0.f;
+  const int last = cnt - 1;
+  if (tid < CL) {
+    const int t = min(tid, last);
+    const size_t at = static_cast<size_t>(tb + t) * a.H + head;
+    const float m_c = w.mc[ch];
+    li[tid] = w.li[at];
+    bc[tid] = w.bc[at];
+    mt[tid] = w.mt[at];
+    gt[tid] = tid < cnt ? expf(static_cast<float>(w.bc[at] + static_cast<double>(m_c) - static_cast<double>(w.mt[at]))) : 0.f;
+  }
+  __syncthreads();
+  constexpr int RT = CL / 16;
+  for (int tile = wave; tile < RT * RT; tile += 4) {
+    const int rt = tile / RT, ct = tile - rt * RT;
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (ct <= rt) {
+      const float* qa = Qs + (16 * rt + l16) * QLD + 4 * lq;
+      const float* kb = Ks + (16 * ct + l16) * QLD + 4 * lq;
+#pragma unroll 4
+      for (int k0 = 0; k0 < DKP; k0 += 16) {
+        const f32x4 a4 = *reinterpret_cast<const f32x4*>(qa + k0), b4 = *reinterpret_cast<const f32x4*>(kb + k0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[e], b4[e], acc, 0, 0, 0);
+      }
+    }
+    const int s = 16 * ct + l16;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int t = 16 * rt + 4 * lq + v;
+      const bool vis = s <= t && t < cnt;
+      As[t * ALD + s] = vis ? acc[v] * expf(static_cast<float>(bc[t] - bc[s]) + li[s] - mt[t]) : 0.f;
+    }
+  }
+  __syncthreads();
+  {
+    const int t = tid % CL, share = tid / CL;
+    constexpr int SH = 256 / CL;
+    float sum = 0.f;
+    for (int s2 = share; s2 < CL; s2 += SH) sum += As[t * ALD + s2];
+    float dot = 0.f;
+    for (int k = share; k < DKP; k += SH) dot = fmaf(Qs[t * QLD + k], ns[k], dot);
+    part[share * CL + t] = fmaf(gt[t], dot, sum);
+  }
+  __syncthreads();
+  if (tid < CL) {
+    constexpr int SH = 256 / CL;
+    float nq = 0.f;
+    for (int sh = 0; sh < SH; ++sh) nq += part[sh * CL + tid];
+    den[tid] = fmaxf(fabsf(nq), expf(-mt[tid])) + 1e-6f;
+  }
+  __syncthreads();
+  for (int tile = wave; tile < RT * (CCOLS / 16); tile += 4) {
+    const int rt = tile / (CCOLS / 16), ct = tile - rt * (CCOLS / 16);
+    f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    const float* aa = As + (16 * rt + l16) * ALD + 4 * lq;
+    const float* vb = Vt + (16 * ct + l16) * VLD + 4 * lq;
+    for (int k0 = 0; k0 < 16 * (rt + 1); k0 += 16) {
+      const f32x4 a4 = *reinterpret_cast<const f32x4*>(aa + k0), b4 = *reinterpret_cast<const f32x4*>(vb + k0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[e], b4[e], acc, 0, 0, 0);
+    }
+    const float g = gt[16 * rt + l16];
+    const float* qa = Qs + (16 * rt + l16) * QLD + 4 * lq;
+    const float* sb = St + (16 * ct + l16) * SLD + 4 * lq;
+#pragma unroll 4
+    for (int k0 = 0; k0 < DKP; k0 += 16) {
+      const f32x4 a4 = *reinterpret_cast<const f32x4*>(qa + k0) * g, b4 = *reinterpret_cast<const f32x4*>(sb + k0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[e], b4[e], acc, 0, 0, 0);
+    }
+    const int c = col0 + 16 * ct + l16;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int t = 16 * rt + 4 * lq + v;
+      if (t < cnt && c < dv) out[static_cast<size_t>(tb + t) * a.H * dv + head * dv + c] = acc[v] / den[t];
+    }
+  }
+}
+
+template <int DKP, int CL> constexpr size_t output_lds() {
+  return sizeof(float) * (2 * CL + 2 * CL * (DKP + 4) + CCOLS * (CL + 4) + CL * (CL + 4) + CCOLS * (DKP + 4) + DKP +
+                          4 * CL + 256);
+}
+template <int DKP, int CL> constexpr size_t local_lds() {
+  return sizeof(float) * (CL * (DKP + 4) + CCOLS * (CL + 4) + CL);
+}
+
+template <typename T, int DKP, int CL>
+int multi_go(const void* qkv, const float* zif, const float* bias_if, const int* cu_q, const int* positions,
+             const int* slot_ids, float* state, float* out, int n_chunks, int n_runs, ScanArgs a, MultiArgs w,
+             hipStream_t s) {
+  static bool allowed = false;
+  if (!allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&mlstm_output_kernel<T, DKP, CL>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(output_lds<DKP, CL>()));
+    if (e == hipSuccess)
+      e = hipFuncSetAttribute(reinterpret_cast<const void*>(&mlstm_local_kernel<T, DKP, CL>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(local_lds<DKP, CL>()));
+    if (e != hipSuccess) return static_cast<int>(e);
+    allowed = true;
+  }
+  const T* rows = static_cast<const T*>(qkv);
+  constexpr size_t lds_local = local_lds<DKP, CL>(), lds_output = output_lds<DKP, CL>();
+  const int slices = (a.dv + CCOLS - 1) / CCOLS;
+  hipLaunchKernelGGL(mlstm_gates_kernel<CL>, dim3(a.H, n_runs), dim3(KVF_WAVE), 0, s, zif, bias_if, cu_q, positions,
+                     slot_ids, state, a, w);
+  hipLaunchKernelGGL((mlstm_local_kernel<T, DKP, CL>), dim3(slices, a.H, n_chunks), dim3(256), lds_local, s,
+                     rows, slot_ids, a, w);
+  const unsigned per_head = static_cast<unsigned>((static_cast<size_t>(a.dk) * a.dv + a.dk + 255) / 256);
+  hipLaunchKernelGGL(mlstm_carry_kernel, dim3(per_head, a.H, n_runs), dim3(256), 0, s, cu_q, positions, slot_ids, state,
+                     a, w);
+  hipLaunchKernelGGL((mlstm_output_kernel<T, DKP, CL>), dim3(slices, a.H, n_chunks), dim3(256), lds_output, s,
+                     rows, slot_ids, out, a, w);
+  return kvf_last_error();
+}
+
+template <typename T>
+int multi_launch(const void* qkv, const float* zif, const float* bias_if, const int* cu_q, const int* positions,
+                 const int* slot_ids, float* state, float* out, int n_chunks, int n_runs, ScanArgs a, MultiArgs w,
+                 hipStream_t s) {
+  if (n_chunks <= 0 || n_runs <= 0) return 0;
+  if (n_chunks > 65535 || n_runs > 65535) return static_cast<int>(hipErrorInvalidValue);
+#define GO(DKP, CL) \
+  return multi_go<T, DKP, CL>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, n_chunks, n_runs, a, w, s)
+  if (a.dk <= 32) GO(32, 64);
+  if (a.dk <= 64) GO(64, 64);
+  if (a.dk <= 128) GO(128, 64);
+  GO(256, 32);
+#undef GO
+}
+
 template <typename T>
 int scan_launch(const void* qkv, const float* zif, const float* bias_if, const int* cu_q, const int* positions,
                 const int* slot_ids, float* state, float* out, int num_seqs, ScanArgs a, hipStream_t s) {
@@ -491,18 +857,23 @@ int out_launch(const float* o, const void* g, int g_stride, const float* w, floa
 // out [tokens, H dv] fp32.  Sequence s owns tokens cu_q[s] .. cu_q[s+1]-1 and slot slot_ids[s]
 // (negative: skipped); it starts from zeros when its first token's position is 0.
 // Runs of fewer than chunk_from tokens are walked token by token (`short_runs`: launch that
-// kernel), runs of at least chunk_from tokens chunk by chunk on the matrix cores (`long_runs`);
-// each kernel leaves the other's sequences alone.
+// kernel), runs of chunk_from to multi_from - 1 tokens chunk by chunk in one kernel (`long_runs`),
+// runs of at least multi_from tokens by the four passes over all chunks at once (n_chunks > 0:
+// `chunks` [n_chunks, 4] and `runs` [n_runs, 3] name them, the other pointers are their scratch);
+// each kernel leaves the others' sequences alone.
 KVF_EXPORT int kvf_mlstm_scan(int dtype, const void* qkv, const float* zif, const float* bias_if,
                               const int* cu_q, const int* positions, const int* slot_ids, float* state,
                               float* out, int num_seqs, int H, int dk, int dv, int row_len, int q_off,
                               int k_off, int v_off, int n_slots, int gate_stride, float cap, float q_scale, int chunk_from,
-                              int short_runs, int long_runs, hipStream_t s) {
+                              int short_runs, int long_runs, int multi_from, int n_chunks, int n_runs,
+                              const int* chunks, const int* runs, float* w_li, float* w_mt, double* w_bc,
+                              float* w_mc, float* w_gl, float* w_W, float* w_un, hipStream_t s) {
   if (H <= 0 || dk <= 0 || dk > 256 || dv <= 0 || !(cap > 0.f) || num_seqs > 65535 || H > 65535 || chunk_from < 1 ||
-      gate_stride < 2 * H)
+      gate_stride < 2 * H || multi_from < chunk_from)
     return static_cast<int>(hipErrorInvalidValue);
   if (dtype != 0 && dtype != 1) return static_cast<int>(hipErrorInvalidValue);
-  const ScanArgs a{H, dk, dv, row_len, q_off, k_off, v_off, num_seqs, n_slots, cap, q_scale, gate_stride, chunk_from};
+  const ScanArgs a{H, dk, dv, row_len, q_off, k_off, v_off, num_seqs, n_slots, cap, q_scale, gate_stride, chunk_from,
+                   multi_from};
   int code = 0;
   if (short_runs)
     code = dtype == 0 ? scan_launch<float>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, num_seqs, a, s)
@@ -510,8 +881,17 @@ KVF_EXPORT int kvf_mlstm_scan(int dtype, const void* qkv, const float* zif, cons
   if (code == 0 && long_runs)
     code = dtype == 0 ? chunk_launch<float>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, num_seqs, a, s)
                       : chunk_launch<bf16_t>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, num_seqs, a, s);
+  if (code == 0 && n_chunks > 0) {
+    if (!chunks || !runs || !w_li || !w_mt || !w_bc || !w_mc || !w_gl || !w_W || !w_un)
+      return static_cast<int>(hipErrorInvalidValue);
+    const MultiArgs w{chunks, runs, w_li, w_mt, w_bc, w_mc, w_gl, w_W, w_un};
+    code = dtype == 0 ? multi_launch<float>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, n_chunks, n_runs, a, w, s)
+                      : multi_launch<bf16_t>(qkv, zif, bias_if, cu_q, positions, slot_ids, state, out, n_chunks, n_runs, a, w, s);
+  }
   return code;
 }
+
+KVF_EXPORT int kvf_mlstm_chunk_len(int dk) { return dk <= 128 ? 64 : 32; }
 
 KVF_EXPORT int kvf_mlstm_out(int dtype, const float* o, const void* g, int g_stride, const float* w, float eps,
                              void* out, int n, int H, int dv, hipStream_t s) {

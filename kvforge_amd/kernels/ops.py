@@ -1115,6 +1115,38 @@ def attn_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
 
 # ------------------------------------------------------------------------------ matrix-memory recurrence
 MLSTM_CHUNK_FROM = 8     # runs of at least so many tokens go chunk by chunk on the matrix cores
+MLSTM_MULTI_FROM = 192   # and runs of at least so many through the passes that take all chunks at once
+
+
+def mlstm_chunk_len(key_dim: int) -> int:
+    """Tokens of a chunk of the matrix-core kernels for heads of this key size."""
+    return 64 if key_dim <= 128 else 32
+
+
+def mlstm_multi_plan(q_lens, key_dim: int, multi_from: int = MLSTM_MULTI_FROM) -> tuple[list[int], list[int]]:
+    """For the runs of at least ``multi_from`` tokens among ``q_lens`` (a step's runs in sequence
+    order): the flat rows ``(sequence, first token, tokens, 0)`` of their chunks and
+    ``(sequence, first chunk, chunks)`` of the runs, as ``mlstm_scan(multi=...)`` wants them."""
+    cl = mlstm_chunk_len(key_dim)
+    chunks: list[int] = []
+    runs: list[int] = []
+    start = 0
+    for seq, q in enumerate(q_lens):
+        if q >= multi_from:
+            first = len(chunks) // 4
+            for t in range(0, q, cl):
+                chunks += [seq, start + t, min(cl, q - t), 0]
+            runs += [seq, first, len(chunks) // 4 - first]
+        start += q
+    return chunks, runs
+
+
+def mlstm_multi_scratch(n_tokens: int, n_chunks: int, heads: int, key_dim: int, value_dim: int) -> dict[str, tuple]:
+    """(shape, dtype) of the scratch tensors the passes over all chunks need, by name."""
+    H, dk, dv = int(heads), int(key_dim), int(value_dim)
+    return {"li": ((n_tokens, H), F32), "mt": ((n_tokens, H), F32), "bc": ((n_tokens, H), torch.float64),
+            "mc": ((n_chunks, H), F32), "gl": ((n_chunks, H), F32), "W": ((n_chunks, H, dk, dv), F32),
+            "un": ((n_chunks, H, dk), F32)}
 
 
 def mlstm_state_floats(heads: int, key_dim: int, value_dim: int) -> int:
@@ -1127,7 +1159,8 @@ def mlstm_scan(rows: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor,
                positions: torch.Tensor, slot_ids: torch.Tensor, state: torch.Tensor, out: torch.Tensor,
                num_seqs: int, heads: int, key_dim: int, value_dim: int, q_off: int, k_off: int,
                v_off: int, cap: float, q_scale: float, chunk_from: int = MLSTM_CHUNK_FROM,
-               short_runs: bool = True, long_runs: bool = True) -> None:
+               short_runs: bool = True, long_runs: bool = True, multi_from: int | None = None,
+               multi: dict | None = None) -> None:
     """The matrix-memory recurrence over every sequence's tokens of this step, from and into the
     sequences' state slots.  ``rows [N, >= ...]``: projected rows holding q (``heads * key_dim``
     elements from column ``q_off``), k (from ``k_off``) and v (``heads * value_dim`` from
@@ -1140,7 +1173,11 @@ def mlstm_scan(rows: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor,
     Two kernels share the work: runs of fewer than ``chunk_from`` tokens are walked token by
     token, longer ones a chunk at a time on the matrix cores (in fp32); ``short_runs`` /
     ``long_runs`` say which of the two are launched (a caller that knows its runs' lengths
-    spares the other launch)."""
+    spares the other launch).  ``multi``: for runs of at least ``multi_from`` tokens, whose chunks
+    are then taken all at once by four passes (gates, every chunk's own contribution, the
+    carry over a run's chunks, the outputs): ``chunks`` ``[n, 4]`` and ``runs`` ``[r, 3]`` (int32,
+    from ``mlstm_multi_plan``) and the scratch tensors of ``mlstm_multi_scratch``; without it no
+    run is that long for the kernels (``multi_from`` is then ignored)."""
     n = rows.shape[0]
     H, dk, dv = int(heads), int(key_dim), int(value_dim)
     _check(rows, "rows", None, (n, None), contiguous=False)
@@ -1164,12 +1201,27 @@ def mlstm_scan(rows: torch.Tensor, gates: torch.Tensor, gate_bias: torch.Tensor,
     _check(out, "out", F32, (n, H * dv))
     if chunk_from < 1:
         raise KernelError(f"mlstm_scan: chunk_from must be positive, got {chunk_from}")
-    f = _fn("mlstm", "kvf_mlstm_scan", [c_int] + [c_void_p] * 8 + [c_int] * 10 + [c_float, c_float] + [c_int] * 3 + [c_void_p])
+    n_chunks = n_runs = 0
+    extra = [None] * 9
+    big = 2**31 - 1
+    if multi is not None:
+        multi_from = MLSTM_MULTI_FROM if multi_from is None else int(multi_from)
+        if multi_from < chunk_from:
+            raise KernelError("mlstm_scan: multi_from must not be below chunk_from")
+        _check(multi["chunks"], "chunks", I32, (None, 4))
+        _check(multi["runs"], "runs", I32, (None, 3))
+        n_chunks, n_runs = multi["chunks"].shape[0], multi["runs"].shape[0]
+        for name, (shape, dtype) in mlstm_multi_scratch(n, n_chunks, H, dk, dv).items():
+            _check(multi[name], name, dtype, shape)
+        extra = [multi[k].data_ptr() for k in ("chunks", "runs", "li", "mt", "bc", "mc", "gl", "W", "un")]
+    f = _fn("mlstm", "kvf_mlstm_scan", [c_int] + [c_void_p] * 8 + [c_int] * 10 + [c_float, c_float] + [c_int] * 6
+            + [c_void_p] * 9 + [c_void_p])
     _ok(f(_tcode(rows.dtype), rows.data_ptr(), gates.data_ptr(), gate_bias.data_ptr(), cu_q.data_ptr(),
           positions.data_ptr(), slot_ids.data_ptr(), state.data_ptr(), out.data_ptr(), int(num_seqs),
           H, dk, dv, rows.stride(0) if n > 1 else rows.shape[1], int(q_off), int(k_off), int(v_off),
           state.shape[0], gates.shape[1], float(cap), float(q_scale), int(chunk_from), 1 if short_runs else 0,
-          1 if long_runs else 0, _stream()), "mlstm_scan")
+          1 if long_runs else 0, multi_from if multi is not None else big, n_chunks, n_runs, *extra,
+          _stream()), "mlstm_scan")
 
 
 def mlstm_out(heads_raw: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float,

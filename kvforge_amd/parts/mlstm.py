@@ -94,6 +94,23 @@ class MatrixLSTM(Mixer):
         return (ops.copies_of(self.w_rows) + ops.copies_of(self.w_o) + ops.copies_of(self.w_gates)
                 + [x for x in (self.gate_bias, self.head_weight) if x is not None])
 
+    def _longest_runs(self, step, n: int) -> dict | None:
+        """What the passes over all chunks at once need for the step's longest runs: the chunk
+        and run tables (made once a step for all layers of this key size, sent along with the
+        batch) and scratch from the step's workspace.  ``None`` when no run is that long."""
+        key = ("mlstm.longest_runs", ops.mlstm_chunk_len(self.dk))
+        plan = step.scratch.get(key)
+        if plan is None:
+            chunks, runs = ops.mlstm_multi_plan(step.q_lens, self.dk)
+            plan = (step.upload_ints(chunks).view(-1, 4), step.upload_ints(runs).view(-1, 3)) if chunks else ()
+            step.scratch[key] = plan
+        if not plan:
+            return None
+        out = {"chunks": plan[0], "runs": plan[1]}
+        for name, (shape, dtype) in ops.mlstm_multi_scratch(n, plan[0].shape[0], self.H, self.dk, self.dv).items():
+            out[name] = step.ws.buf("mlstm_multi_" + name, shape, dtype)
+        return out
+
     def forward(self, x, step, layer: LayerState, residual) -> None:
         """``x``: normalised activations."""
         if layer.state is None:
@@ -109,11 +126,12 @@ class MatrixLSTM(Mixer):
         raw = ws.buf("mlstm_raw", (n, H * dv), torch.float32)
         # which of the two kernels have work is known from the runs' lengths (all ones in a
         # captured step of single tokens, so a replay launches what the capture launched)
-        long_runs = any(q >= ops.MLSTM_CHUNK_FROM for q in step.q_lens)
+        long_runs = any(ops.MLSTM_CHUNK_FROM <= q < ops.MLSTM_MULTI_FROM for q in step.q_lens)
         short_runs = any(q < ops.MLSTM_CHUNK_FROM for q in step.q_lens)
         ops.mlstm_scan(rows, gates, self.gate_bias, step.cu_q, step.positions, step.slot_ids,
                        layer.state, raw, step.n_seqs, H, dk, dv, 0, H * dk, 2 * H * dk,
-                       self.gate_cap, float(dk) ** -0.5, short_runs=short_runs, long_runs=long_runs)
+                       self.gate_cap, float(dk) ** -0.5, short_runs=short_runs, long_runs=long_runs,
+                       multi=self._longest_runs(step, n))
         heads = ws.buf("mlstm_heads", (n, H * dv), act)
         g0 = 2 * H * dk + H * dv
         ops.mlstm_out(raw, rows[:, g0:g0 + H * dv], self.head_weight, self.norm_eps, heads, H, dv)

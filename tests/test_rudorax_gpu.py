@@ -231,6 +231,47 @@ def test_matrix_memory_over_many_chunks(dtype, H, dk, dv):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,dk,dv", [(2, 40, 72), (1, 136, 64), (1, 256, 40), (3, 16, 130)])
+def test_matrix_memory_with_all_chunks_at_once(dtype, H, dk, dv):
+    """Three sequences in two steps: the longest runs go through the passes that take all
+    chunks at once, beside a run for the one-kernel chunks and single tokens; every run carries
+    on from the state that another kernel left in its slot."""
+    cap = 15.0
+    lens = {"a": 300, "b": 210, "c": 150}
+    cols = 2 * H * dk + H * dv
+    data = {r: (rand(n, cols, seed=i + dk).to(dtype), rand(n, 2 * H, seed=i + 9, scale=3.0)) for i, (r, n) in enumerate(lens.items())}
+    bias = torch.cat([torch.full((H,), -1.0), torch.full((H,), 5.0)])
+    want = {}
+    for r, (rows, z) in data.items():
+        x = rows.float()
+        want[r] = scan_reference(x[:, :H * dk], x[:, H * dk:2 * H * dk], x[:, 2 * H * dk:], z[:, :H], z[:, H:], bias, cap, H, dk, dv)
+    state = torch.full((3, ops().mlstm_state_floats(H, dk, dv)), 3.0, device=DEV)
+    slot = {"a": 1, "b": 2, "c": 0}
+    got = {r: [] for r in lens}
+    multi_from = 100
+    for step in ([("a", 0, 131), ("b", 0, 1), ("c", 0, 40)], [("b", 1, 210), ("c", 40, 150), ("a", 131, 132)],
+                 [("a", 132, 300)]):
+        rows = torch.cat([data[r][0][a:b] for r, a, b in step]).to(DEV)
+        z = torch.cat([data[r][1][a:b] for r, a, b in step]).to(DEV)
+        q_lens = [b - a for _, a, b in step]
+        chunks, runs = ops().mlstm_multi_plan(q_lens, dk, multi_from)
+        multi = {"chunks": i32(chunks).view(-1, 4), "runs": i32(runs).view(-1, 3)}
+        for name, (shape, dt) in ops().mlstm_multi_scratch(rows.shape[0], len(chunks) // 4, H, dk, dv).items():
+            multi[name] = torch.full(shape, float("nan"), dtype=dt, device=DEV)
+        out = torch.full((rows.shape[0], H * dv), 5.0, device=DEV)
+        ops().mlstm_scan(rows, z, bias.to(DEV), i32([0] + list(np.cumsum(q_lens))),
+                         torch.cat([torch.arange(a, b) for _, a, b in step]).int().to(DEV),
+                         i32([slot[r] for r, _, _ in step]), state, out, len(step), H, dk, dv, 0, H * dk, 2 * H * dk,
+                         cap, dk ** -0.5, multi_from=multi_from, multi=multi)
+        off = 0
+        for (r, a, b) in step:
+            got[r].append(out[off:off + b - a].cpu())
+            off += b - a
+    for r in lens:
+        torch.testing.assert_close(torch.cat(got[r]), want[r], atol=3e-4, rtol=3e-4)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_heads_normed_weighted_and_gated(dtype):
     H, dv, n, eps = 3, 40, 5, 1e-3
     raw, w = rand(n, H * dv, seed=1, scale=4.0), 1.0 + rand(H * dv, seed=2, scale=0.2)
