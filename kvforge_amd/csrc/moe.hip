@@ -211,29 +211,40 @@ __global__ __launch_bounds__(256) void moe_up_kernel(const bf16_t* __restrict__ 
     for (int g = 0; g < GW; ++g) acc[r][g] = f32x4{0.f, 0.f, 0.f, 0.f};
   const uint4* wbase = wt + (static_cast<size_t>(e) * groups + g_first) * S * KVF_WAVE + lane;
   const int s_full = K / 32;   // steps whose 32 elements all lie inside a row
-  auto step = [&](int s) {
-    bf16x8 b[RT];
+  // the fragments of a step are asked for two steps ahead of the matrix instructions that use
+  // them: three sets of registers take turns
+  bf16x8 xb[3][RT], wb[3][GW];
+  auto load = [&](int s, bf16x8 (&xs)[RT], bf16x8 (&ws)[GW]) {
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
       uint4 xf = make_uint4(0u, 0u, 0u, 0u);
       if (xr[r] && (s < s_full || 32 * s + 8 * c + 8 <= K)) xf = *reinterpret_cast<const uint4*>(xr[r] + 32 * s);
-      b[r] = __builtin_bit_cast(bf16x8, xf);
+      xs[r] = __builtin_bit_cast(bf16x8, xf);
     }
 #pragma unroll
-    for (int g = 0; g < GW; ++g) {   // ff is a multiple of 32, so the groups come in whole fours
-      const bf16x8 wf = __builtin_bit_cast(bf16x8, wbase[(static_cast<size_t>(g) * S + s) * KVF_WAVE]);
-#pragma unroll
-      for (int r = 0; r < RT; ++r) acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, b[r], acc[r][g], 0, 0, 0);
-    }
+    for (int g = 0; g < GW; ++g)   // ff is a multiple of 32, so the groups come in whole fours
+      ws[g] = __builtin_bit_cast(bf16x8, wbase[(static_cast<size_t>(g) * S + s) * KVF_WAVE]);
   };
-  int s = 0;
-  for (; s + 4 <= S; s += 4) {
-    step(s);
-    step(s + 1);
-    step(s + 2);
-    step(s + 3);
+  auto mma = [&](const bf16x8 (&xs)[RT], const bf16x8 (&ws)[GW]) {
+#pragma unroll
+    for (int g = 0; g < GW; ++g)
+#pragma unroll
+      for (int r = 0; r < RT; ++r) acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ws[g], xs[r], acc[r][g], 0, 0, 0);
+  };
+  load(0, xb[0], wb[0]);
+  if (S > 1) load(1, xb[1], wb[1]);
+  for (int s = 0; s < S; s += 3) {
+    if (s + 2 < S) load(s + 2, xb[2], wb[2]);
+    mma(xb[0], wb[0]);
+    if (s + 1 < S) {
+      if (s + 3 < S) load(s + 3, xb[0], wb[0]);
+      mma(xb[1], wb[1]);
+    }
+    if (s + 2 < S) {
+      if (s + 4 < S) load(s + 4, xb[1], wb[1]);
+      mma(xb[2], wb[2]);
+    }
   }
-  for (; s < S; ++s) step(s);
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
     if (16 * r + j >= rows) continue;
@@ -279,29 +290,38 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const bf16_t* __restrict_
   int goff[GW];
 #pragma unroll
   for (int g = 0; g < GW; ++g) goff[g] = min(g, groups - 1 - g_first);
-  auto step = [&](int s) {
-    bf16x8 b[RT];
+  bf16x8 xb[3][RT], wb[3][GW];
+  auto load = [&](int s, bf16x8 (&xs)[RT], bf16x8 (&ws)[GW]) {
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
       uint4 af = make_uint4(0u, 0u, 0u, 0u);
       if (ar[r]) af = *reinterpret_cast<const uint4*>(ar[r] + 32 * s);
-      b[r] = __builtin_bit_cast(bf16x8, af);
+      xs[r] = __builtin_bit_cast(bf16x8, af);
     }
 #pragma unroll
-    for (int g = 0; g < GW; ++g) {   // a group past the last is read as the last and not stored
-      const bf16x8 wf = __builtin_bit_cast(bf16x8, wbase[(static_cast<size_t>(goff[g]) * S_all + s) * KVF_WAVE]);
-#pragma unroll
-      for (int r = 0; r < RT; ++r) acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, b[r], acc[r][g], 0, 0, 0);
-    }
+    for (int g = 0; g < GW; ++g)   // a group past the last is read as the last and not stored
+      ws[g] = __builtin_bit_cast(bf16x8, wbase[(static_cast<size_t>(goff[g]) * S_all + s) * KVF_WAVE]);
   };
-  int s = 0;
-  for (; s + 4 <= S; s += 4) {
-    step(s);
-    step(s + 1);
-    step(s + 2);
-    step(s + 3);
+  auto mma = [&](const bf16x8 (&xs)[RT], const bf16x8 (&ws)[GW]) {
+#pragma unroll
+    for (int g = 0; g < GW; ++g)
+#pragma unroll
+      for (int r = 0; r < RT; ++r) acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ws[g], xs[r], acc[r][g], 0, 0, 0);
+  };
+  load(0, xb[0], wb[0]);
+  if (S > 1) load(1, xb[1], wb[1]);
+  for (int s = 0; s < S; s += 3) {
+    if (s + 2 < S) load(s + 2, xb[2], wb[2]);
+    mma(xb[0], wb[0]);
+    if (s + 1 < S) {
+      if (s + 3 < S) load(s + 3, xb[0], wb[0]);
+      mma(xb[1], wb[1]);
+    }
+    if (s + 2 < S) {
+      if (s + 4 < S) load(s + 4, xb[1], wb[1]);
+      mma(xb[2], wb[2]);
+    }
   }
-  for (; s < S; ++s) step(s);
 #pragma unroll
   for (int r = 0; r < RT; ++r) {
     if (16 * r + j >= rows) continue;
