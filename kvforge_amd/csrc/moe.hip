@@ -135,6 +135,7 @@ __global__ __launch_bounds__(256) void moe_identity_kernel(float* __restrict__ x
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 constexpr int PLAN_MAX_EXPERTS = 512;
+constexpr int PREFETCH_SETS = 3;   // sets of operand registers in flight in the grouped products
 
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ sel, int pairs, int E,
                                                         int* __restrict__ where, int* __restrict__ order,
@@ -211,9 +212,10 @@ __global__ __launch_bounds__(256) void moe_up_kernel(const bf16_t* __restrict__ 
     for (int g = 0; g < GW; ++g) acc[r][g] = f32x4{0.f, 0.f, 0.f, 0.f};
   const uint4* wbase = wt + (static_cast<size_t>(e) * groups + g_first) * S * KVF_WAVE + lane;
   const int s_full = K / 32;   // steps whose 32 elements all lie inside a row
-  // the fragments of a step are asked for two steps ahead of the matrix instructions that use
-  // them: three sets of registers take turns
-  bf16x8 xb[3][RT], wb[3][GW];
+  // the fragments of a step are asked for NB - 1 steps ahead of the matrix instructions that use
+  // them: NB sets of registers take turns
+  constexpr int NB = PREFETCH_SETS;
+  bf16x8 xb[NB][RT], wb[NB][GW];
   auto load = [&](int s, bf16x8 (&xs)[RT], bf16x8 (&ws)[GW]) {
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
@@ -231,18 +233,16 @@ __global__ __launch_bounds__(256) void moe_up_kernel(const bf16_t* __restrict__ 
 #pragma unroll
       for (int r = 0; r < RT; ++r) acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ws[g], xs[r], acc[r][g], 0, 0, 0);
   };
-  load(0, xb[0], wb[0]);
-  if (S > 1) load(1, xb[1], wb[1]);
-  for (int s = 0; s < S; s += 3) {
-    if (s + 2 < S) load(s + 2, xb[2], wb[2]);
-    mma(xb[0], wb[0]);
-    if (s + 1 < S) {
-      if (s + 3 < S) load(s + 3, xb[0], wb[0]);
-      mma(xb[1], wb[1]);
-    }
-    if (s + 2 < S) {
-      if (s + 4 < S) load(s + 4, xb[1], wb[1]);
-      mma(xb[2], wb[2]);
+#pragma unroll
+  for (int i = 0; i < NB - 1; ++i)
+    if (i < S) load(i, xb[i], wb[i]);
+  for (int s = 0; s < S; s += NB) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      if (s + i < S) {
+        if (s + i + NB - 1 < S) load(s + i + NB - 1, xb[(i + NB - 1) % NB], wb[(i + NB - 1) % NB]);
+        mma(xb[i], wb[i]);
+      }
     }
   }
 #pragma unroll
@@ -290,7 +290,8 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const bf16_t* __restrict_
   int goff[GW];
 #pragma unroll
   for (int g = 0; g < GW; ++g) goff[g] = min(g, groups - 1 - g_first);
-  bf16x8 xb[3][RT], wb[3][GW];
+  constexpr int NB = PREFETCH_SETS;
+  bf16x8 xb[NB][RT], wb[NB][GW];
   auto load = [&](int s, bf16x8 (&xs)[RT], bf16x8 (&ws)[GW]) {
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
@@ -308,18 +309,16 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const bf16_t* __restrict_
 #pragma unroll
       for (int r = 0; r < RT; ++r) acc[r][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ws[g], xs[r], acc[r][g], 0, 0, 0);
   };
-  load(0, xb[0], wb[0]);
-  if (S > 1) load(1, xb[1], wb[1]);
-  for (int s = 0; s < S; s += 3) {
-    if (s + 2 < S) load(s + 2, xb[2], wb[2]);
-    mma(xb[0], wb[0]);
-    if (s + 1 < S) {
-      if (s + 3 < S) load(s + 3, xb[0], wb[0]);
-      mma(xb[1], wb[1]);
-    }
-    if (s + 2 < S) {
-      if (s + 4 < S) load(s + 4, xb[1], wb[1]);
-      mma(xb[2], wb[2]);
+#pragma unroll
+  for (int i = 0; i < NB - 1; ++i)
+    if (i < S) load(i, xb[i], wb[i]);
+  for (int s = 0; s < S; s += NB) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      if (s + i < S) {
+        if (s + i + NB - 1 < S) load(s + i + NB - 1, xb[(i + NB - 1) % NB], wb[(i + NB - 1) % NB]);
+        mma(xb[i], wb[i]);
+      }
     }
   }
 #pragma unroll
