@@ -151,6 +151,54 @@ KVF_EXPORT int kvf_rmsnorm_bf16(float* x, const int* rows, const void* delta, in
   return rmsnorm_launch<bf16_t, bf16_t>(x, rows, delta, w, wf, eps, out, m, h, xr, s);
 }
 
+// Two norms of the same row in one pass: y1 = v r w1 and y2 = v r w2 with v = x (+ delta, which is
+// then written back to x) and r = rsqrt(mean(v^2) + eps): for a block whose two sublayers each
+// have a norm of their own over the same stream.  Weights are fp32.
+template <typename T, typename D>
+__global__ void rmsnorm_pair_kernel(float* __restrict__ x, const D* __restrict__ delta,
+                                    const float* __restrict__ w1, const float* __restrict__ w2, float eps,
+                                    T* __restrict__ out1, T* __restrict__ out2, int h) {
+  __shared__ float scratch[16];
+  const size_t m = blockIdx.x;
+  float* xr = x + m * h;
+  const D* dr = delta ? delta + m * h : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < h; i += blockDim.x) {
+    float v = xr[i];
+    if (dr) {
+      v += Elem<D>::load(dr + i);
+      xr[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float r = rsqrtf(ss / static_cast<float>(h) + eps);
+  for (int i = threadIdx.x; i < h; i += blockDim.x) {
+    const float v = xr[i] * r;   // the sum where it was written back (by this same thread)
+    Elem<T>::store(out1 + m * h + i, v * w1[i]);
+    Elem<T>::store(out2 + m * h + i, v * w2[i]);
+  }
+}
+template <typename T, typename D>
+static int rmsnorm_pair_launch(float* x, const void* delta, const float* w1, const float* w2, float eps, void* o1,
+                               void* o2, int m, int h, hipStream_t s) {
+  if (m <= 0) return 0;
+  const int threads = h >= 1024 ? 256 : (h >= 256 ? 128 : 64);
+  hipLaunchKernelGGL((rmsnorm_pair_kernel<T, D>), dim3(m), dim3(threads), 0, s, x, static_cast<const D*>(delta), w1, w2,
+                     eps, static_cast<T*>(o1), static_cast<T*>(o2), h);
+  return kvf_last_error();
+}
+KVF_EXPORT int kvf_rmsnorm_pair_f32(float* x, const void* delta, int delta_f32, const float* w1, const float* w2,
+                                    float eps, void* o1, void* o2, int m, int h, hipStream_t s) {
+  (void)delta_f32;
+  return rmsnorm_pair_launch<float, float>(x, delta, w1, w2, eps, o1, o2, m, h, s);
+}
+KVF_EXPORT int kvf_rmsnorm_pair_bf16(float* x, const void* delta, int delta_f32, const float* w1, const float* w2,
+                                     float eps, void* o1, void* o2, int m, int h, hipStream_t s) {
+  if (delta_f32) return rmsnorm_pair_launch<bf16_t, float>(x, delta, w1, w2, eps, o1, o2, m, h, s);
+  return rmsnorm_pair_launch<bf16_t, bf16_t>(x, delta, w1, w2, eps, o1, o2, m, h, s);
+}
+
 // ----------------------------------------------------------------------------- residual sum
 // x[m] += delta[m] in fp32 (x is the residual stream, delta a product in T).
 template <typename T>

@@ -155,6 +155,28 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor | None, eps: float, out: torch
           m, h, xr, _stream()), "rmsnorm")
 
 
+def rmsnorm_pair(x: torch.Tensor, weight1: torch.Tensor, weight2: torch.Tensor, eps: float,
+                 out1: torch.Tensor, out2: torch.Tensor, add: torch.Tensor | None = None) -> None:
+    """Two RMS norms of the same rows in one pass: ``out1 = y * weight1`` and ``out2 = y * weight2``
+    with ``y = v * rsqrt(mean(v^2) + eps)`` and ``v = x`` (``+ add``, a sum still owed to ``x``, which
+    is then left in ``x``).  Weights fp32 ``[h]``; outputs of one type."""
+    _check(x, "x", F32, (None, None))
+    m, h = x.shape
+    _check(weight1, "weight1", F32, (h,))
+    _check(weight2, "weight2", F32, (h,))
+    _check(out1, "out1", None, (m, h))
+    _check(out2, "out2", out1.dtype, (m, h))
+    if add is not None:
+        _check(add, "add", None, (m, h))
+        if add.dtype not in (F32, out1.dtype):
+            raise KernelError(f"rmsnorm_pair: add must be float32 or {out1.dtype}, got {add.dtype}")
+    f = _fn("elementwise", f"kvf_rmsnorm_pair_{_suffix(out1.dtype)}",
+            [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p])
+    _ok(f(x.data_ptr(), add.data_ptr() if add is not None else None,
+          1 if add is not None and add.dtype == F32 else 0, weight1.data_ptr(), weight2.data_ptr(), float(eps),
+          out1.data_ptr(), out2.data_ptr(), m, h, _stream()), "rmsnorm_pair")
+
+
 def add_rows(x: torch.Tensor, delta: torch.Tensor) -> None:
     """``x += delta`` for the fp32 residual stream ``x`` and a product ``delta`` of equal shape."""
     _check(x, "x", F32, (None, None))

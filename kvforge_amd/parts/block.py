@@ -85,6 +85,15 @@ class ParallelBlock(Block):
     def parts(self) -> list[Part]:
         return [p for p in (self.norm, self.ffn_norm, self.mixer, self.ffn, self.after) if p is not None]
 
+    def _norms_pair(self) -> bool:
+        """Whether the two norms are RMS norms with fp32 weight vectors and one eps, which one
+        kernel then takes together."""
+        a, b = self.norm, self.ffn_norm
+        return (b is not None and type(a).forward is type(b).forward
+                and all(isinstance(getattr(n, "weight", None), torch.Tensor) and n.weight.dtype == torch.float32
+                        for n in (a, b))
+                and getattr(a, "eps", None) == getattr(b, "eps", 0.0))
+
     def weight_specs(self) -> dict[str, WeightSpec]:
         out = super().weight_specs()
         if self.shift_name is not None:
@@ -116,10 +125,16 @@ class ParallelBlock(Block):
             hs = step.ws.buf("parallel_shifted", shape, step.act_dtype)
             ops.norm_shift(residual, self.norm.weight, self.mu, layer.state, step.slot_ids,
                            step.seq_of_token, step.cu_q, step.positions, self.norm.eps, h, hs)
+        elif self._norms_pair():
+            # two RMS norms of the same stream: one pass over it, two weights
+            hs = h
+            h = step.ws.buf("parallel_normed_ffn", shape, step.act_dtype)
+            ops.rmsnorm_pair(residual, self.norm.weight, self.ffn_norm.weight, self.norm.eps, hs, h,
+                             add=step.take_owed(residual))
         else:
             self.norm.forward(residual, h, add=step.take_owed(residual))
             hs = h
-        if self.ffn_norm is not None:
+        if self.ffn_norm is not None and not (self.mu is None and self._norms_pair()):
             # of the same stream as the mixer's norm: taken before the mixer adds to it
             h = step.ws.buf("parallel_normed_ffn", shape, step.act_dtype)
             self.ffn_norm.forward(residual, h)
